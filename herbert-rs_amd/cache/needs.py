@@ -7,10 +7,13 @@ import torch
 
 @dataclass(frozen=True)
 class KVNeed:
-    """Keys and values of every position, or of the last `window` positions only."""
+    """Keys and values of every position, or of the last `window` positions only. `values` False:
+    rows of keys alone (a mixer whose values are a part of its key rows, as an attention over one
+    shared latent a token has them); the pool is then half the size and the view's `v` is None."""
     kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    values: bool = True
 
 
 @dataclass(frozen=True)

@@ -43,9 +43,12 @@ class KVGroup:
         self.need = need
         self.entries = list(entries)
         self.pages = FreeList(n_pages, "page")
-        self.pages_per_slot = pages_for(max_positions)
+        # a slot's table has a place for every page a sequence can hold at once: the model's positions, and
+        # without a window (whose slots give pages back as they grow) no more than the pool has
+        self.pages_per_slot = pages_for(max_positions) if need.window else min(pages_for(max_positions), n_pages)
+        self.halves = 2 if need.values else 1
         # (one page and one slot more than sequences can hold: the padding page and the padding slot)
-        self.pool = torch.zeros((len(self.entries), 2, n_pages + 1, need.kv_heads, PAGE_TOKENS,
+        self.pool = torch.zeros((len(self.entries), self.halves, n_pages + 1, need.kv_heads, PAGE_TOKENS,
                                  need.head_dim), dtype=dtype, device=device)
         self.table_host = np.full((n_slots, self.pages_per_slot), -1, dtype=np.int32)
         # entries of the device table that are not held point at page 0: a kernel never reads
@@ -61,7 +64,9 @@ class KVGroup:
         i = self.entries.index(entry)
         n_pages = self.pool.shape[2]         # (with the padding page)
         k = self.pool[i, 0]
-        v = self.pool[i, 1].view(n_pages, self.need.kv_heads, self.need.head_dim, PAGE_TOKENS)
+        v = None
+        if self.need.values:
+            v = self.pool[i, 1].view(n_pages, self.need.kv_heads, self.need.head_dim, PAGE_TOKENS)
         return LayerKV(k, v, self.table, PAGE_TOKENS, int(self.need.window or 0))
 
     def pages_missing(self, slot, new_length):
@@ -196,7 +201,7 @@ class Cache:
         total = 0
         for need, entries in by_need.items():
             if isinstance(need, KVNeed):
-                total += entries * 2 * n_pages * PAGE_TOKENS * need.kv_heads * need.head_dim * element
+                total += entries * (2 if need.values else 1) * n_pages * PAGE_TOKENS * need.kv_heads * need.head_dim * element
             elif isinstance(need, StateNeed):
                 per_slot = 1
                 for d in need.shape:

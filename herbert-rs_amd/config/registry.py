@@ -3,7 +3,7 @@
 An entry holds the configuration class, the builder of the model's
 specification, how its checkpoints spell tensor names (weights/names.py) and
 how a chat turn is written for it. The name is `architectures[0]` of
-config.json, or `model_type` when that is absent; when config.json names
+config.json (or its `architecture`, a string), or `model_type` when that is absent; when config.json names
 neither, the architecture registered with `default=True` is taken (the
 reference selects by `model_type` alone and takes "qwen3" when the key is
 missing: crates/core/src/config.rs:95-102,184-185,261-263). An unknown name
@@ -93,6 +93,8 @@ def resolve_architecture(raw):
     """The Architecture that a config dict names."""
     load_plugins()
     archs = raw.get("architectures")
+    if not (isinstance(archs, list) and archs) and isinstance(raw.get("architecture"), str):
+        archs = [raw["architecture"]]           # (some families name theirs under a key of its own)
     if isinstance(archs, list) and archs:
         name = archs[0]
         if name in _ARCHITECTURES:

@@ -453,3 +453,78 @@ extern "C" int hb_fill_u32(void* p, uint32_t value, size_t n, hipStream_t stream
     HB_CHECK_LAUNCH("fill_u32");
     return 0;
 }
+
+// ---------------------------------------------------------------- layer norm
+// y[r, :] = (x[src(r), :] - mean) / sqrt(var + eps) * w, var = the mean of the squared deviations
+// (two passes over the row: the deviations are taken from the mean, not from sums of squares);
+// no bias. y may be x itself (float32, no gather): every element is read by the thread that writes it,
+// and all reads of a pass are done before the block's sum is.
+// DELTA: the row is first x + mult * delta (the sum of a layer's parts joins the residual stream),
+// written back to x, and that sum is what is normed: one kernel between two layers.
+template <class TOut, bool DELTA>
+__global__ void layernorm_kernel(float* x, const float* __restrict__ delta, float mult,
+                                 const float* __restrict__ w, TOut* y, const int* __restrict__ rows, int H,
+                                 float eps) {
+    __shared__ float red[16];
+    const int r = blockIdx.x;
+    const size_t src = (size_t)(rows ? rows[r] : r) * H;
+    float* in = x + src;
+    TOut* out = y + (size_t)r * H;
+    float s = 0.f;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        float v = in[i];
+        if (DELTA) {
+            v = fmaf(mult, delta[src + i], v);
+            in[i] = v;
+        }
+        s += v;
+    }
+    const float mean = hb_block_sum(s, red) / (float)H;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        const float d = in[i] - mean;
+        ss += d * d;
+    }
+    ss = hb_block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+    if (y == nullptr) return;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = hb_from_float<TOut>((in[i] - mean) * inv * w[i]);
+}
+
+// delta may be null (a plain layer norm). With delta, rows must be null and x is updated in place;
+// y null: only the sum is wanted (after the last layer).
+extern "C" int hb_layernorm(float* x, const float* delta, float mult, const float* w, void* y, int y_dtype,
+                            const int* rows, int R, int H, float eps, hipStream_t stream) {
+    HB_REQUIRE(R > 0 && H > 0, "layernorm: empty input (R=%d, H=%d)", R, H);
+    HB_REQUIRE(y_dtype == HB_F32 || y_dtype == HB_BF16, "layernorm: unknown output dtype %d", y_dtype);
+    HB_REQUIRE(delta == nullptr || rows == nullptr, "layernorm: rows are not gathered while a sum is added");
+    HB_REQUIRE(y != nullptr || delta != nullptr, "layernorm: nothing to do");
+    const int threads = H >= 1024 ? 256 : H >= 256 ? 128 : 64;
+    if (delta) {
+        if (y_dtype == HB_F32)
+            layernorm_kernel<float, true><<<R, threads, 0, stream>>>(x, delta, mult, w, (float*)y, rows, H, eps);
+        else
+            layernorm_kernel<bf16, true><<<R, threads, 0, stream>>>(x, delta, mult, w, (bf16*)y, rows, H, eps);
+    } else {
+        if (y_dtype == HB_F32)
+            layernorm_kernel<float, false><<<R, threads, 0, stream>>>(x, nullptr, 0.f, w, (float*)y, rows, H, eps);
+        else
+            layernorm_kernel<bf16, false><<<R, threads, 0, stream>>>(x, nullptr, 0.f, w, (bf16*)y, rows, H, eps);
+    }
+    HB_CHECK_LAUNCH("layernorm");
+    return 0;
+}
+
+// ---------------------------------------------------------------- x = x * s (float32, in place)
+__global__ void scale_kernel(float* x, float s, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        x[i] *= s;
+}
+
+extern "C" int hb_scale(float* x, float s, size_t n, hipStream_t stream) {
+    HB_REQUIRE(n > 0, "scale: empty input");
+    const size_t blocks = (n + 255) / 256;
+    scale_kernel<<<(unsigned)(blocks > 4096 ? 4096 : blocks), 256, 0, stream>>>(x, s, n);
+    HB_CHECK_LAUNCH("scale");
+    return 0;
+}

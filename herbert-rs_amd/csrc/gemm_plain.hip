@@ -17,7 +17,11 @@ HB_MODULE_ERROR_SLOT()
 template <class TA, class TW, class TC, bool ACCUM>
 __global__ void __launch_bounds__(256)
 gemm_plain_kernel(const TA* __restrict__ A, const TW* __restrict__ W, TC* __restrict__ C, int M, int N,
-                  int K, int lda, int ldw, int ldc) {
+                  int K, int lda, int ldw, int ldc, size_t batch_a, size_t batch_w, size_t batch_c) {
+    // (blockIdx.z: one of a batch of products whose operands lie batch_* elements apart)
+    A += blockIdx.z * batch_a;
+    W += blockIdx.z * batch_w;
+    C += blockIdx.z * batch_c;
     __shared__ float As[TILE_K][TILE_M + 1];
     __shared__ float Ws[TILE_K][TILE_N + 1];
     const int tid = threadIdx.x;
@@ -80,14 +84,15 @@ gemm_plain_kernel(const TA* __restrict__ A, const TW* __restrict__ W, TC* __rest
 
 template <class TA, class TW, class TC>
 static void launch(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldw, int ldc,
-                   int accumulate, hipStream_t stream) {
-    dim3 grid((N + TILE_N - 1) / TILE_N, (M + TILE_M - 1) / TILE_M);
+                   int accumulate, hipStream_t stream, int batch = 1, size_t batch_a = 0, size_t batch_w = 0,
+                   size_t batch_c = 0) {
+    dim3 grid((N + TILE_N - 1) / TILE_N, (M + TILE_M - 1) / TILE_M, batch);
     if (accumulate)
         gemm_plain_kernel<TA, TW, TC, true><<<grid, 256, 0, stream>>>(
-            (const TA*)A, (const TW*)W, (TC*)C, M, N, K, lda, ldw, ldc);
+            (const TA*)A, (const TW*)W, (TC*)C, M, N, K, lda, ldw, ldc, batch_a, batch_w, batch_c);
     else
         gemm_plain_kernel<TA, TW, TC, false><<<grid, 256, 0, stream>>>(
-            (const TA*)A, (const TW*)W, (TC*)C, M, N, K, lda, ldw, ldc);
+            (const TA*)A, (const TW*)W, (TC*)C, M, N, K, lda, ldw, ldc, batch_a, batch_w, batch_c);
 }
 
 // C[M, N] (+)= A[M, K] * W[N, K]^T with row strides lda, ldw, ldc (in elements).
@@ -110,5 +115,32 @@ extern "C" int hb_gemm_plain(const void* A, int a_dtype, const void* W, int w_dt
         default: HB_REQUIRE(false, "gemm: unknown dtypes (%d, %d, %d)", a_dtype, w_dtype, c_dtype);
     }
     HB_CHECK_LAUNCH("gemm_plain");
+    return 0;
+}
+
+// A batch of such products in one launch: product b reads A + b * batch_a, W + b * batch_w and writes
+// C + b * batch_c (elements). Heads that each have a matrix of their own are such a batch: the row
+// strides let every head's columns lie inside rows that all heads share.
+extern "C" int hb_gemm_plain_batched(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype,
+                                     int M, int N, int K, int lda, int ldw, int ldc, int batch, size_t batch_a,
+                                     size_t batch_w, size_t batch_c, hipStream_t stream) {
+    HB_REQUIRE(M > 0 && N > 0 && K > 0 && batch > 0, "gemm: empty problem (M=%d, N=%d, K=%d, batch=%d)", M, N, K, batch);
+    HB_REQUIRE(lda >= K && ldw >= K && ldc >= N, "gemm: a row stride is smaller than its row");
+    HB_REQUIRE((M + TILE_M - 1) / TILE_M <= 65535 && batch <= 65535, "gemm: M=%d or batch=%d exceeds the grid", M, batch);
+    const int key = a_dtype * 4 + w_dtype * 2 + c_dtype;
+#define HB_BATCHED(TA, TW, TC) launch<TA, TW, TC>(A, W, C, M, N, K, lda, ldw, ldc, 0, stream, batch, batch_a, batch_w, batch_c)
+    switch (key) {
+        case 0: HB_BATCHED(float, float, float); break;
+        case 1: HB_BATCHED(float, float, bf16); break;
+        case 2: HB_BATCHED(float, bf16, float); break;
+        case 3: HB_BATCHED(float, bf16, bf16); break;
+        case 4: HB_BATCHED(bf16, float, float); break;
+        case 5: HB_BATCHED(bf16, float, bf16); break;
+        case 6: HB_BATCHED(bf16, bf16, float); break;
+        case 7: HB_BATCHED(bf16, bf16, bf16); break;
+        default: HB_REQUIRE(false, "gemm: unknown dtypes (%d, %d, %d)", a_dtype, w_dtype, c_dtype);
+    }
+#undef HB_BATCHED
+    HB_CHECK_LAUNCH("gemm_plain_batched");
     return 0;
 }

@@ -1,0 +1,284 @@
+// A feed-forward of many small experts of which each token uses a few.
+//   route     the router's logits (+ bias) of a token -> its `top` experts (largest logits, the
+//             lower index of equals) and their weights, the softmax over the chosen logits only
+//   group     the (token, choice) pairs in the order of their experts, so that an expert's rows
+//             are consecutive, and a list of row tiles (expert, first row, rows) of fixed length
+//   products  a tile's rows times its expert's matrix, float32 sums over k ascending by one
+//             thread each (plain), whatever else is in the batch
+//   activate  g = min(gate, limit), u = clamp(up, -limit, limit): y = g sigmoid(alpha g) (u + 1)
+//   combine   a token's rows weighted and summed in the order of its choices, added to the output
+// Nothing here asks the host: the grids depend on the step's size only, so a step can be recorded
+// and replayed.
+#include "common.h"
+#include <math.h>
+
+HB_MODULE_ERROR_SLOT()
+
+#define MOE_TILE_M 64
+#define MOE_TILE_N 64
+#define MOE_TILE_K 16
+#define MOE_MAX_E_PER_LANE 16
+
+// ------------------------------------------------------------------------ route
+// One wave a token; lane l holds the logits of experts l, l + 64, ...
+__global__ void __launch_bounds__(HB_WAVE)
+moe_route_kernel(const float* __restrict__ logits, const float* __restrict__ bias, int* __restrict__ chosen,
+                 float* __restrict__ weight, int E, int top) {
+    const int t = blockIdx.x, lane = threadIdx.x;
+    float z[MOE_MAX_E_PER_LANE];
+#pragma unroll
+    for (int i = 0; i < MOE_MAX_E_PER_LANE; ++i) {
+        const int e = lane + HB_WAVE * i;
+        z[i] = e < E ? logits[(size_t)t * E + e] + (bias ? bias[e] : 0.f) : -INFINITY;
+    }
+    float first = 0.f, sum = 0.f;
+    for (int j = 0; j < top; ++j) {
+        float best = -INFINITY;
+        int at = 0x7fffffff;
+#pragma unroll
+        for (int i = 0; i < MOE_MAX_E_PER_LANE; ++i) {
+            const int e = lane + HB_WAVE * i;
+            if (e < E && (z[i] > best || (z[i] == best && e < at))) {
+                best = z[i];
+                at = e;
+            }
+        }
+#pragma unroll
+        for (int off = HB_WAVE / 2; off > 0; off >>= 1) {
+            const float ob = __shfl_xor(best, off, HB_WAVE);
+            const int oa = __shfl_xor(at, off, HB_WAVE);
+            if (ob > best || (ob == best && oa < at)) {
+                best = ob;
+                at = oa;
+            }
+        }
+        if (j == 0) first = best;                    // the first choice is the largest
+        const float p = expf(best - first);
+        sum += p;
+        if (lane == j % HB_WAVE) {                   // (the lane that divides it below)
+            chosen[(size_t)t * top + j] = at;
+            weight[(size_t)t * top + j] = p;
+        }
+#pragma unroll
+        for (int i = 0; i < MOE_MAX_E_PER_LANE; ++i)
+            if (lane + HB_WAVE * i == at) z[i] = -INFINITY;
+    }
+    for (int j = lane; j < top; j += HB_WAVE) weight[(size_t)t * top + j] /= sum;
+}
+
+// ------------------------------------------------------------------------ group
+__global__ void moe_count_kernel(const int* __restrict__ chosen, int* __restrict__ counts, int A) {
+    __shared__ int red[16];
+    const int e = blockIdx.x;
+    int n = 0;
+    for (int a = threadIdx.x; a < A; a += blockDim.x) n += chosen[a] == e;
+    for (int off = HB_WAVE / 2; off > 0; off >>= 1) n += __shfl_xor(n, off, HB_WAVE);
+    if ((threadIdx.x & (HB_WAVE - 1)) == 0) red[threadIdx.x / HB_WAVE] = n;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int total = 0;
+        for (int w = 0; w < (int)(blockDim.x / HB_WAVE); ++w) total += red[w];
+        counts[e] = total;
+    }
+}
+
+// Block e < E: the pairs of expert e, in the order of the pairs, to rows [first, first + count) and
+// the expert's tiles into the list; block E: the list's unused end. order[row] = pair,
+// row_of[pair] = row.
+__global__ void __launch_bounds__(256)
+moe_place_kernel(const int* __restrict__ chosen, const int* __restrict__ counts, int* __restrict__ order,
+                 int* __restrict__ row_of, int* __restrict__ tile_expert, int* __restrict__ tile_row0,
+                 int* __restrict__ tile_rows, int A, int E, int max_tiles) {
+    __shared__ int wave_n[4];
+    __shared__ int base;
+    const int e = blockIdx.x;
+    int first = 0, tile0 = 0;
+    for (int i = 0; i < (e < E ? e : E); ++i) {
+        first += counts[i];
+        tile0 += (counts[i] + MOE_TILE_M - 1) / MOE_TILE_M;
+    }
+    if (e == E) {
+        for (int i = tile0 + threadIdx.x; i < max_tiles; i += blockDim.x) tile_expert[i] = -1;
+        return;
+    }
+    const int count = counts[e];
+    for (int i = threadIdx.x; i * MOE_TILE_M < count; i += blockDim.x) {
+        tile_expert[tile0 + i] = e;
+        tile_row0[tile0 + i] = first + i * MOE_TILE_M;
+        tile_rows[tile0 + i] = count - i * MOE_TILE_M < MOE_TILE_M ? count - i * MOE_TILE_M : MOE_TILE_M;
+    }
+    if (threadIdx.x == 0) base = first;
+    __syncthreads();
+    const int lane = threadIdx.x & (HB_WAVE - 1), wave = threadIdx.x / HB_WAVE;
+    for (int a0 = 0; a0 < A; a0 += 256) {
+        const int a = a0 + threadIdx.x;
+        const bool hit = a < A && chosen[a] == e;
+        const unsigned long long mask = __ballot(hit);
+        if (lane == 0) wave_n[wave] = __popcll(mask);
+        __syncthreads();
+        int before = 0;
+        for (int w = 0; w < wave; ++w) before += wave_n[w];
+        if (hit) {
+            const int row = base + before + __popcll(mask & ((1ull << lane) - 1ull));
+            order[row] = a;
+            row_of[a] = row;
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) base += wave_n[0] + wave_n[1] + wave_n[2] + wave_n[3];
+        __syncthreads();
+    }
+}
+
+extern "C" int hb_moe_route(const float* logits, const float* bias, int* chosen, float* weight, int* counts,
+                            int* order, int* row_of, int* tile_expert, int* tile_row0, int* tile_rows, int T, int E,
+                            int top, int max_tiles, hipStream_t stream) {
+    HB_REQUIRE(T > 0 && E > 0 && top > 0 && top <= E, "moe: %d of %d experts for %d tokens", top, E, T);
+    HB_REQUIRE(E <= HB_WAVE * MOE_MAX_E_PER_LANE, "moe: %d experts, the router takes up to %d", E, HB_WAVE * MOE_MAX_E_PER_LANE);
+    const long long A = (long long)T * top;
+    HB_REQUIRE(A < (1ll << 30), "moe: too many (token, expert) pairs");
+    HB_REQUIRE(max_tiles >= (A + MOE_TILE_M - 1) / MOE_TILE_M + E, "moe: the tile list is too short");
+    moe_route_kernel<<<T, HB_WAVE, 0, stream>>>(logits, bias, chosen, weight, E, top);
+    HB_CHECK_LAUNCH("moe_route");
+    moe_count_kernel<<<E, 256, 0, stream>>>(chosen, counts, (int)A);
+    HB_CHECK_LAUNCH("moe_count");
+    moe_place_kernel<<<E + 1, 256, 0, stream>>>(chosen, counts, order, row_of, tile_expert, tile_row0, tile_rows, (int)A, E, max_tiles);
+    HB_CHECK_LAUNCH("moe_place");
+    return 0;
+}
+
+// ------------------------------------------------------------------------ products, plain
+// C[row, n] = sum_k A[src(row), k] * W[e][n, k] for the rows of every tile; src(row) = order[row] / top
+// (the token's row of the activations) if `top` > 0, else the row itself.
+template <class TA, class TW, class TC>
+__global__ void __launch_bounds__(256)
+moe_gemm_plain_kernel(const TA* __restrict__ A, const TW* __restrict__ W, TC* __restrict__ C,
+                      const int* __restrict__ order, const int* __restrict__ tile_expert,
+                      const int* __restrict__ tile_row0, const int* __restrict__ tile_rows, int top, int N, int K) {
+    __shared__ float As[MOE_TILE_K][MOE_TILE_M + 1];
+    __shared__ float Ws[MOE_TILE_K][MOE_TILE_N + 1];
+    __shared__ int src[MOE_TILE_M];
+    const int e = tile_expert[blockIdx.y];
+    if (e < 0) return;
+    const int row0 = tile_row0[blockIdx.y], rows = tile_rows[blockIdx.y];
+    const int tid = threadIdx.x;
+    const int tx = tid % 16, ty = tid / 16;
+    const int n0 = blockIdx.x * MOE_TILE_N;
+    const TW* We = W + (size_t)e * N * K;
+    if (tid < MOE_TILE_M) src[tid] = tid < rows ? (top > 0 ? order[row0 + tid] / top : row0 + tid) : -1;
+    __syncthreads();
+
+    float acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+
+    for (int k0 = 0; k0 < K; k0 += MOE_TILE_K) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int el = tid + i * 256;
+            const int kk = el % MOE_TILE_K, rr = el / MOE_TILE_K;
+            const int k = k0 + kk, n = n0 + rr;
+            As[kk][rr] = (src[rr] >= 0 && k < K) ? hb_to_float(A[(size_t)src[rr] * K + k]) : 0.f;
+            Ws[kk][rr] = (n < N && k < K) ? hb_to_float(We[(size_t)n * K + k]) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < MOE_TILE_K; ++kk) {
+            float a[4], w[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[i] = As[kk][ty + 16 * i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) w[j] = Ws[kk][tx + 16 * j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = ty + 16 * i;
+        if (r >= rows) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + tx + 16 * j;
+            if (n < N) C[(size_t)(row0 + r) * N + n] = hb_from_float<TC>(acc[i][j]);
+        }
+    }
+}
+
+// A [rows, K] (the tokens' rows if top > 0, else one row a pair), W [E, N, K], C [pairs, N].
+extern "C" int hb_moe_gemm_plain(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype,
+                                 const int* order, const int* tile_expert, const int* tile_row0,
+                                 const int* tile_rows, int max_tiles, int top, int N, int K, hipStream_t stream) {
+    HB_REQUIRE(N > 0 && K > 0 && max_tiles > 0 && max_tiles <= 65535 * 16, "moe product: empty or too large");
+    HB_REQUIRE(max_tiles <= 65535, "moe product: %d row tiles exceed the grid", max_tiles);
+    const dim3 grid((N + MOE_TILE_N - 1) / MOE_TILE_N, max_tiles);
+    const int key = a_dtype * 4 + w_dtype * 2 + c_dtype;
+#define HB_MOE(TA, TW, TC)                                                                                        \
+    moe_gemm_plain_kernel<TA, TW, TC><<<grid, 256, 0, stream>>>((const TA*)A, (const TW*)W, (TC*)C, order,        \
+                                                                tile_expert, tile_row0, tile_rows, top, N, K)
+    switch (key) {
+        case 0: HB_MOE(float, float, float); break;
+        case 2: HB_MOE(float, bf16, float); break;
+        case 4: HB_MOE(bf16, float, float); break;
+        case 6: HB_MOE(bf16, bf16, float); break;
+        default: HB_REQUIRE(false, "moe product: dtypes (%d, %d, %d) are not built (the sums are float32)", a_dtype, w_dtype, c_dtype);
+    }
+#undef HB_MOE
+    HB_CHECK_LAUNCH("moe_gemm_plain");
+    return 0;
+}
+
+// ------------------------------------------------------------------------ activate
+// gu [pairs, 2 F] float32 (gate columns, then up columns) -> act [pairs, F]
+template <class TOut>
+__global__ void moe_activate_kernel(const float* __restrict__ gu, TOut* __restrict__ act, int F, size_t total,
+                                    float limit, float alpha) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t r = i / F;
+        const int n = (int)(i % F);
+        const float g = fminf(gu[r * 2 * F + n], limit);
+        const float u = fminf(fmaxf(gu[r * 2 * F + F + n], -limit), limit);
+        act[i] = hb_from_float<TOut>(g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+    }
+}
+
+extern "C" int hb_moe_activate(const float* gu, void* act, int act_dtype, int rows, int F, float limit, float alpha,
+                               hipStream_t stream) {
+    HB_REQUIRE(rows > 0 && F > 0, "moe activation: empty input");
+    const size_t total = (size_t)rows * F;
+    const size_t blocks = (total + 255) / 256;
+    const unsigned grid = (unsigned)(blocks > 8192 ? 8192 : blocks);
+    if (act_dtype == HB_F32)
+        moe_activate_kernel<float><<<grid, 256, 0, stream>>>(gu, (float*)act, F, total, limit, alpha);
+    else if (act_dtype == HB_BF16)
+        moe_activate_kernel<bf16><<<grid, 256, 0, stream>>>(gu, (bf16*)act, F, total, limit, alpha);
+    else
+        HB_REQUIRE(false, "moe activation: unknown output dtype %d", act_dtype);
+    HB_CHECK_LAUNCH("moe_activate");
+    return 0;
+}
+
+// ------------------------------------------------------------------------ combine
+// x[t, :] += sum_j weight[t, j] * y[row_of[t * top + j], :]    (float32, j ascending)
+__global__ void moe_combine_kernel(const float* __restrict__ y, const float* __restrict__ weight,
+                                   const int* __restrict__ row_of, float* __restrict__ x, int top, int H) {
+    const int t = blockIdx.x;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        float s = 0.f;
+        for (int j = 0; j < top; ++j)
+            s = fmaf(weight[(size_t)t * top + j], y[(size_t)row_of[(size_t)t * top + j] * H + i], s);
+        x[(size_t)t * H + i] += s;
+    }
+}
+
+extern "C" int hb_moe_combine(const float* y, const float* weight, const int* row_of, float* x, int T, int top, int H,
+                              hipStream_t stream) {
+    HB_REQUIRE(T > 0 && top > 0 && H > 0, "moe combine: empty input");
+    moe_combine_kernel<<<T, H >= 1024 ? 256 : 64, 0, stream>>>(y, weight, row_of, x, top, H);
+    HB_CHECK_LAUNCH("moe_combine");
+    return 0;
+}

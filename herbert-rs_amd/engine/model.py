@@ -36,7 +36,9 @@ class Model:
         self.blocks = []
         for layer in spec.layers:
             mixer = build("mixer", layer.mixer, shared=self.shared)
-            ffn = build("feed_forward", layer.feed_forward, shared=self.shared)
+            ffn = None          # (a layer may have no feed-forward, if its arrangement allows that)
+            if layer.feed_forward is not None:
+                ffn = build("feed_forward", layer.feed_forward, shared=self.shared)
             norms = {role: build("norm", ns) for role, ns in layer.norms.items()}
             self.blocks.append(build("block", layer.block, mixer=mixer, feed_forward=ffn, norms=norms))
         final_norm = build("norm", spec.final_norm)
@@ -110,6 +112,7 @@ class Model:
             ctx.owns_cache = e.cache is None
             # the norm that the residual stream meets after this block, for parts that can prepare it
             ctx.norm_after_block = None
+            ctx.next_block = self.blocks[self.schedule[i + 1].layer] if i + 1 < len(self.schedule) else None
             if i + 1 < len(self.schedule):
                 first_norm = getattr(self.blocks[self.schedule[i + 1].layer], "first_norm", None)
                 if first_norm is not None:

@@ -26,9 +26,27 @@ SIGNATURES = {
                                   _I, _I, _I, _I, _F, _I, _I, ctypes.c_size_t, _P],
         "hb_swiglu": [_P, _P, _I, _I, _I, _P],
         "hb_fill_u32": [_P, _U32, _SZ, _P],
+        "hb_layernorm": [_P, _P, _F, _P, _P, _I, _P, _I, _I, _F, _P],
+        "hb_scale": [_P, _F, _SZ, _P],
     },
     "gemm_plain": {
         "hb_gemm_plain": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P],
+        "hb_gemm_plain_batched": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _SZ, _SZ, _SZ, _P],
+    },
+    "recurrent": {
+        "hb_conv_silu": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I, _I, _P],
+        "hb_gated_delta": [_P, _I, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
+        "hb_gated_head_norm": [_P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _P],
+    },
+    "attention_latent": {
+        "hb_latent_write": [_P, _I, _P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
+        "hb_latent_attention_plain": [_P, _P, _P, _I, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P],
+    },
+    "moe": {
+        "hb_moe_route": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
+        "hb_moe_gemm_plain": [_P, _I, _P, _I, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _P],
+        "hb_moe_activate": [_P, _P, _I, _I, _I, _F, _F, _P],
+        "hb_moe_combine": [_P, _P, _P, _P, _I, _I, _I, _P],
     },
     "attention_plain": {
         "hb_attention_plain": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],

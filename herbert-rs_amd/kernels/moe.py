@@ -1,0 +1,89 @@
+"""Host side of the routed feed-forward's kernels (csrc/moe.hip): routing and grouping, the products
+of an expert's rows with its matrices, the activation, and the weighted sum."""
+import torch
+
+from ..errors import BackendError
+from . import lib
+from .ops import _check, _ptr, _stream, dtype_code
+
+TILE_M = 64
+MAX_EXPERTS = 1024
+
+
+def max_tiles(pairs, experts):
+    """The length of the list of row tiles for that many (token, expert) pairs."""
+    return (pairs + TILE_M - 1) // TILE_M + experts
+
+
+class Routing:
+    """The buffers that routing fills for a step of T tokens: chosen int32 [T, top], weight f32 [T, top],
+    order / row_of int32 [T top], the tiles' lists."""
+
+    def __init__(self, ints, weight, T, E, top):
+        A, tiles = T * top, max_tiles(T * top, E)
+        need = 3 * A + E + 3 * tiles
+        if ints.numel() < need or ints.dtype != torch.int32:
+            raise BackendError("routing: the int32 buffer is too small")
+        self.T, self.E, self.top, self.tiles = T, E, top, tiles
+        o = 0
+        self.chosen, o = ints[o:o + A], o + A
+        self.order, o = ints[o:o + A], o + A
+        self.row_of, o = ints[o:o + A], o + A
+        self.counts, o = ints[o:o + E], o + E
+        self.tile_expert, o = ints[o:o + tiles], o + tiles
+        self.tile_row0, o = ints[o:o + tiles], o + tiles
+        self.tile_rows, o = ints[o:o + tiles], o + tiles
+        self.weight = weight
+
+    @staticmethod
+    def ints_needed(T, E, top):
+        return 3 * T * top + E + 3 * max_tiles(T * top, E)
+
+
+def route(logits, bias, routing):
+    """logits f32 [T, E] (+ bias f32 [E]) -> routing (see Routing)."""
+    r = routing
+    _check(logits, "logits", torch.float32, (r.T, r.E))
+    if bias is not None:
+        _check(bias, "bias", torch.float32, (r.E,))
+    _check(r.weight, "weight", torch.float32, (r.T, r.top))
+    if r.E > MAX_EXPERTS or not 0 < r.top <= r.E:
+        raise BackendError(f"routing: {r.top} of {r.E} experts")
+    lib.call("moe", "hb_moe_route", logits.data_ptr(), _ptr(bias), r.chosen.data_ptr(), r.weight.data_ptr(),
+             r.counts.data_ptr(), r.order.data_ptr(), r.row_of.data_ptr(), r.tile_expert.data_ptr(),
+             r.tile_row0.data_ptr(), r.tile_rows.data_ptr(), r.T, r.E, r.top, r.tiles, _stream())
+
+
+def gemm_plain(a, w, c, routing, gather):
+    """c[row] = a[src(row)] @ w[expert of row]^T for every pair's row; w [E, N, K]; a [T, K] with
+    gather (src = the pair's token) or [pairs, K]; c f32 [pairs, N]."""
+    r = routing
+    E, N, K = w.shape
+    _check(w, "w", None, (r.E, N, K))
+    _check(a, "a", None, (r.T if gather else r.T * r.top, K))
+    _check(c, "c", torch.float32, (r.T * r.top, N))
+    lib.call("moe", "hb_moe_gemm_plain", a.data_ptr(), dtype_code(a), w.data_ptr(), dtype_code(w), c.data_ptr(),
+             dtype_code(c), r.order.data_ptr(), r.tile_expert.data_ptr(), r.tile_row0.data_ptr(),
+             r.tile_rows.data_ptr(), r.tiles, r.top if gather else 0, N, K, _stream())
+
+
+def activate(gu, act, limit, alpha):
+    """gu f32 [pairs, 2 F] (gate | up) -> act [pairs, F] = g sigmoid(alpha g) (u + 1) with g = min(gate,
+    limit), u = clamp(up, -limit, limit)."""
+    rows, two_f = gu.shape
+    _check(gu, "gate_up", torch.float32, (rows, two_f))
+    if two_f % 2:
+        raise BackendError("moe activation: the input's width must be even")
+    _check(act, "act", None, (rows, two_f // 2))
+    lib.call("moe", "hb_moe_activate", gu.data_ptr(), act.data_ptr(), dtype_code(act), rows, two_f // 2, float(limit),
+             float(alpha), _stream())
+
+
+def combine(y, routing, x):
+    """x[t] += sum_j weight[t, j] * y[row of pair (t, j)]; y f32 [pairs, H], x f32 [T, H]."""
+    r = routing
+    H = x.shape[1]
+    _check(y, "y", torch.float32, (r.T * r.top, H))
+    _check(x, "x", torch.float32, (r.T, H))
+    lib.call("moe", "hb_moe_combine", y.data_ptr(), r.weight.data_ptr(), r.row_of.data_ptr(), x.data_ptr(), r.T,
+             r.top, H, _stream())

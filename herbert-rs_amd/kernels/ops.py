@@ -350,3 +350,56 @@ def force_tokens(logits, rows, tokens):
     both = torch.tensor([list(map(int, rows)), list(map(int, tokens))], dtype=torch.int32, device=logits.device)
     lib.call("sampling", "hb_force_tokens", logits.data_ptr(), V, R, V, both[0].data_ptr(), both[1].data_ptr(),
              len(rows), _stream())
+
+
+def layernorm(x, weight, out, eps, rows=None, delta=None, mult=1.0):
+    """out[r] = (x[r] - mean) / sqrt(var + eps) * weight, var the mean of the squared deviations; x f32
+    [T, H] (rows int32: only these, gathered), out f32 or the compute dtype, and it may be x itself.
+    delta f32 [T, H]: x becomes x + mult * delta first, in place, and that sum is normed (no rows then);
+    out None with a delta: only the sum."""
+    _check(x, "x", torch.float32, (None, None))
+    H = x.shape[1]
+    _check(weight, "weight", torch.float32, (H,))
+    if rows is not None:
+        _check(rows, "rows", torch.int32, (None,))
+        R = rows.shape[0]
+    else:
+        R = x.shape[0]
+    if delta is not None:
+        _check(delta, "delta", torch.float32, tuple(x.shape))
+        if rows is not None:
+            raise BackendError("layernorm: rows are not gathered while a sum is added")
+    elif out is None:
+        raise BackendError("layernorm: nothing to do")
+    if out is not None:
+        _check(out, "out", None, (R, H))
+    lib.call("elementwise", "hb_layernorm", x.data_ptr(), _ptr(delta), float(mult), weight.data_ptr(), _ptr(out),
+             dtype_code(out) if out is not None else F32, _ptr(rows), R, H, float(eps), _stream())
+
+
+def scale(x, factor):
+    """x *= factor in place; x float32."""
+    _check(x, "x", torch.float32)
+    lib.call("elementwise", "hb_scale", x.data_ptr(), float(factor), x.numel(), _stream())
+
+
+def gemm_plain_batched(a, w, c, M, N, K, lda, ldw, ldc, batch, batch_a, batch_w, batch_c):
+    """`batch` products c_b[M, N] = a_b[M, K] @ w_b[N, K]^T in one launch, float32 arithmetic: product b
+    reads a + b * batch_a, w + b * batch_w and writes c + b * batch_c (elements), rows lda / ldw / ldc
+    elements apart. The caller's tensors must hold every element that this addresses."""
+    for t, name, ld, rows, cols, step in ((a, "a", lda, M, K, batch_a), (w, "w", ldw, N, K, batch_w),
+                                          (c, "c", ldc, M, N, batch_c)):
+        _check(t, name)
+        last = (batch - 1) * step + (rows - 1) * ld + cols
+        if ld < cols or last > t.numel():
+            raise BackendError(f"batched gemm: {name} of {t.numel()} elements does not hold the batch (needs {last})")
+    lib.call("gemm_plain", "hb_gemm_plain_batched", a.data_ptr(), dtype_code(a), w.data_ptr(), dtype_code(w),
+             c.data_ptr(), dtype_code(c), M, N, K, lda, ldw, ldc, batch, batch_a, batch_w, batch_c, _stream())
+
+
+def layernorm_free_sum(x, delta, mult):
+    """x += mult * delta, float32 in place (the layer norm's kernel without its norm)."""
+    _check(x, "x", torch.float32, (None, None))
+    _check(delta, "delta", torch.float32, tuple(x.shape))
+    lib.call("elementwise", "hb_layernorm", x.data_ptr(), delta.data_ptr(), float(mult), None, None, F32, None,
+             x.shape[0], x.shape[1], 0.0, _stream())

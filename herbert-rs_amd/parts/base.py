@@ -149,6 +149,9 @@ class StepContext:
     left: Any = None
     norm_after_block: Any = None     # set by the model: (first norm of the next entry's block, entry)
     logits_out: Any = None           # where the head is to write, if the caller owns the logits
+    next_block: Any = None           # set by the model: the block of the schedule's next entry, or None
+    # (x, delta, mult): a sum that a block has left for the next block's norm to add to x (x += mult * delta)
+    pending_sum: Any = None
 
     def leave_norm(self, linear, x):
         """For a part, just before `linear` adds its last product into x: a NormedRows that product

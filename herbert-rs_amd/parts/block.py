@@ -1,10 +1,16 @@
 """How a layer's parts are arranged.
 
+"parallel": with h = norm(x), x += mult * (mixer(h) + feed_forward(h)): one norm, both parts read it,
+and their sum joins the residual stream times a constant.
+
 "prenorm": x += mixer(norm_input(x)); x += feed_forward(norm_post_mixer(x)), the
 arrangement of the reference's two-norm layer
 (crates/backends/backend_common/src/generic_layer.rs:1149-1151, 1234-1236,
 1246-1248, 1272-1274).
 """
+import torch
+
+from ..kernels import ops
 from .base import Part
 from .registry import register
 
@@ -54,3 +60,55 @@ class PreNormBlock(Part):
             return
         ctx.handed = None
         part.forward(ctx, norm.forward(ctx, x), x)
+
+
+@register("block", "parallel")
+class ParallelBlock(Part):
+    """x <- x + mult * (mixer(h) + feed_forward(h)) with h = norm(x). The parts add their outputs, as they
+    always do, to float32 rows of their own (cleared first) instead of to x. Where the next layer is such
+    a block with a norm that can take a sum on, the sum is left for that norm's kernel, which adds it to x
+    and norms the result in one pass; otherwise it is added here."""
+    graph_safe = True
+
+    norm_roles = ("input",)
+
+    def __init__(self, mixer, feed_forward, norms, mult=1.0, fuse_sum=True):
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        if "input" not in norms:
+            raise ValueError("parallel block needs the norm 'input'")
+        self.norm = norms["input"]
+        self.mult = float(mult)
+        self.fuse_sum = bool(fuse_sum)
+
+    def parts(self):
+        return [self.norm, self.mixer] + ([self.feed_forward] if self.feed_forward is not None else [])
+
+    def first_norm(self):
+        return self.norm
+
+    def takes_sum(self):
+        """True if this block's norm adds a sum that the block before left (ctx.pending_sum)."""
+        return self.fuse_sum and getattr(self.norm, "adds_sum", False)
+
+    def forward(self, ctx, x):
+        pending, ctx.pending_sum = ctx.pending_sum, None
+        if pending is not None and pending[0].data_ptr() == x.data_ptr() and self.takes_sum():
+            h = self.norm.forward(ctx, x, delta=pending[1], mult=pending[2])
+        else:
+            if pending is not None:
+                ops.layernorm_free_sum(x, pending[1], pending[2])
+            h = self.norm.forward(ctx, x)
+        # the two parts' outputs meet in rows of their own (free again: the norm above has taken the sum
+        # of the layer before)
+        total = ctx.rt.buffer("parallel_sum", tuple(x.shape), torch.float32)
+        ops.fill_u32(total, 0)
+        ctx.handed = ctx.norm_ahead = None
+        self.mixer.forward(ctx, h, total)
+        if self.feed_forward is not None:
+            self.feed_forward.forward(ctx, h, total)
+        nxt = ctx.next_block
+        if isinstance(nxt, ParallelBlock) and nxt.takes_sum():
+            ctx.pending_sum = (x, total, self.mult)
+        else:
+            ops.layernorm_free_sum(x, total, self.mult)

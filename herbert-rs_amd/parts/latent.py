@@ -1,0 +1,98 @@
+"""Attention whose keys and values come from one low-rank latent a token.
+
+From the normed rows h: q = W_q h, a head's [dim unrotated | rot_dim rotated]; W_dkv h has kv_rank +
+rot_dim rows: the first kv_rank, RMS-normed with a weight, are the latent c, the last rot_dim, rotated,
+are one key part that all heads share. Head n's key is [W_uk,n c | that part], its value W_uv,n c; the
+score is the dot product of query and key times `scale`, causal, plain softmax; the head's output is
+multiplied by sigmoid(W_g h)_n and the heads go through W_o.
+
+Only c and the rotated part are cached, one row a token ([kv_rank + rot_dim], no values of their
+own). The kernels never build a head's keys or values: the query's unrotated part is taken through
+W_uk,n^T first (kv_rank numbers), scores and weighted sums then run on the cached rows themselves,
+one shared "key head" for all query heads, and the summed latents go through W_uv,n afterwards.
+Scores, softmax and the weighted sums are float32 in either mode.
+"""
+import torch
+
+from ..cache import KVNeed
+from ..kernels import latent, ops
+from ..weights import TensorNeed
+from .base import Part
+from .linear import Linear
+from .registry import register
+
+
+@register("mixer", "latent_attention")
+class LatentAttention(Part):
+    graph_safe = True
+
+    def __init__(self, hidden_size, heads, dim, rot_dim, vdim, kv_rank, scale, eps, position, names, shared=None):
+        """names: q, dkv, dkv_norm, uk, uv, g (None: no output gate), o -> tensor names. position: the
+        spec of a rotation (its rotary_dims <= rot_dim entries of the rotated part are rotated)."""
+        self.hidden_size, self.heads = int(hidden_size), int(heads)
+        self.dim, self.rot_dim, self.vdim, self.rank = int(dim), int(rot_dim), int(vdim), int(kv_rank)
+        self.scale, self.eps = float(scale), float(eps)
+        self.names = dict(names)
+        self.position = shared.position(position)
+        if self.rank > latent.MAX_RANK or self.rot_dim > latent.MAX_ROT:
+            raise ValueError(f"the latent attention's kernels take a latent of up to {latent.MAX_RANK} + "
+                             f"{latent.MAX_ROT}, not {self.rank} + {self.rot_dim}")
+
+    @property
+    def row(self):
+        return self.rank + self.rot_dim
+
+    def tensor_needs(self):
+        n, W, H = self.names, self.hidden_size, self.heads
+        needs = {n["q"]: TensorNeed((H * (self.dim + self.rot_dim), W)), n["dkv"]: TensorNeed((self.row, W)),
+                 n["dkv_norm"]: TensorNeed((self.rank,), "scale"), n["uk"]: TensorNeed((H * self.dim, self.rank)),
+                 n["uv"]: TensorNeed((H * self.vdim, self.rank)), n["o"]: TensorNeed((W, H * self.vdim))}
+        if n.get("g"):
+            needs[n["g"]] = TensorNeed((H, W))
+        return needs
+
+    def cache_need(self):
+        return KVNeed(1, self.row, None, values=False)
+
+    def load(self, tensors, rt):
+        n, H = self.names, self.heads
+        rows = [tensors[n["q"]].to(rt.device), tensors[n["dkv"]].to(rt.device)]
+        self.gated = bool(n.get("g"))
+        if self.gated:
+            rows.append(tensors[n["g"]].to(rt.device))
+        # one projection [q | latent and shared key part | gate]
+        self.proj = Linear(rt.weight(torch.cat(rows, 0)), scratch=rt.scratch)
+        self.q_width = H * (self.dim + self.rot_dim)
+        self.width = self.q_width + self.row + (H if self.gated else 0)
+        self.norm_w = rt.weight(tensors[n["dkv_norm"]], matrix=False)
+        # W_uk a head, transposed: [H, rank, dim], so that q' = W_uk,n^T q_n is a product with rows of k = dim
+        uk = rt.weight(tensors[n["uk"]]).view(H, self.dim, self.rank)
+        self.uk_t = uk.transpose(1, 2).contiguous()
+        self.uv = rt.weight(tensors[n["uv"]]).view(H, self.vdim, self.rank).contiguous()
+        self.o = Linear(rt.weight(tensors[n["o"]]), scratch=rt.scratch)
+        rot = self.position.rotation_rates()
+        self.inv_freq, self.rot_dims = (None, 0) if rot is None else rot
+        if self.rot_dims > self.rot_dim:
+            raise ValueError(f"{self.rot_dims} rotated entries do not fit the rotated part of {self.rot_dim}")
+
+    def forward(self, ctx, y, x):
+        rt, H = ctx.rt, self.heads
+        T = y.shape[0]
+        kv = ctx.cache.kv_view(ctx.cache_entry)
+        proj = rt.buffer("latent_proj", (T, self.width), torch.float32)
+        self.proj.forward(y, proj)
+        q_full = rt.buffer("latent_q_full", (T, H * self.row), torch.float32)
+        latent.latent_write(proj, 0, self.q_width, self.norm_w, q_full, self.inv_freq, ctx.meta, kv, H, self.dim,
+                            self.rank, self.rot_dim, self.rot_dims, self.eps, write_cache=ctx.owns_cache)
+        # q'[t, n, :] = W_uk,n^T q[t, n, :dim]: a product a head, all in one launch
+        ops.gemm_plain_batched(proj, self.uk_t, q_full, T, self.rank, self.dim, self.width, self.dim,
+                               H * self.row, H, self.dim + self.rot_dim, self.rank * self.dim, self.row)
+        mixed = rt.buffer("latent_mixed", (T, H * self.rank))
+        latent.latent_attention_plain(q_full, ctx.meta, kv, mixed, proj if self.gated else None,
+                                      self.q_width + self.row, H, self.rank, self.rot_dim, self.scale)
+        # a head's summed latents through its W_uv
+        attn = rt.buffer("latent_attn", (T, H * self.vdim))
+        ops.gemm_plain_batched(mixed, self.uv, attn, T, self.vdim, self.rank, H * self.rank, self.rank, H * self.vdim,
+                               H, self.rank, self.vdim * self.rank, self.vdim)
+        left = ctx.leave_norm(self.o, x)
+        self.o.forward(attn, x, accumulate=True, leave=None if left is None else left.leave())

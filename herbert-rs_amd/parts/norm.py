@@ -1,4 +1,4 @@
-"""RMSNorm as the reference computes it (crates/backends/backend_common/src/kernels.rs:54-64):
+"""Norms of the residual stream. RMSNorm as the reference computes it (crates/backends/backend_common/src/kernels.rs:54-64):
 y = x / sqrt(mean(x^2) + eps) * w, the weight used as stored (not 1 + w)."""
 from ..kernels import ops
 from ..weights import TensorNeed
@@ -28,3 +28,36 @@ class RMSNorm(Part):
         y = ctx.rt.buffer(name, (n, self.size))
         ops.rmsnorm(x, self.w, y, self.eps, rows)
         return y
+
+
+@register("norm", "layernorm")
+class LayerNorm(Part):
+    """y = (x - mean) / sqrt(var + eps) * w with var the mean of the squared deviations; a weight and
+    no bias. Not of the form x * w / rms(x), so no product can finish it (`hands_on` stays off); what
+    it can take on instead is the sum that joins the residual stream just before it
+    (`forward(..., delta=, mult=)`: x <- x + mult * delta, then the norm of that, one kernel)."""
+    graph_safe = True
+    adds_sum = True      # forward(..., delta=, mult=) adds a sum to x on the way
+
+    def __init__(self, size, eps, weight):
+        self.size = int(size)
+        self.eps = float(eps)
+        self.weight_name = weight
+        self.w = None
+
+    def tensor_needs(self):
+        return {self.weight_name: TensorNeed((self.size,), "scale")}
+
+    def load(self, tensors, rt):
+        self.w = rt.weight(tensors[self.weight_name], matrix=False)
+
+    def forward(self, ctx, x, rows=None, name="normed", delta=None, mult=1.0):
+        n = x.shape[0] if rows is None else rows.shape[0]
+        y = ctx.rt.buffer(name, (n, self.size))
+        ops.layernorm(x, self.w, y, self.eps, rows, delta=delta, mult=mult)
+        return y
+
+    def forward_in_place(self, ctx, x):
+        """x <- norm(x), float32: for a norm that is part of the residual stream itself."""
+        ops.layernorm(x, self.w, x, self.eps)
+        return x

@@ -27,12 +27,18 @@ class NoPosition(Part):
     def rotation(self):
         return None
 
+    def rotation_rates(self):
+        return None
+
 
 @register("position", "rope")
 class RotaryHalfSplit(Part):
     graph_safe = True
 
-    def __init__(self, theta, rotary_dims, max_positions, scaling=None):
+    def __init__(self, theta, rotary_dims, max_positions, scaling=None, tables=True):
+        """tables False: no cos / sin tables are built (`rotation()` is then None); a mixer whose kernels
+        take the angles from `rotation_rates()` needs none, and its positions have no bound but the cache's."""
+        self.tables = bool(tables)
         if rotary_dims % 2:
             raise ValueError("rotary_dims must be even")
         self.theta = float(theta)
@@ -65,10 +71,19 @@ class RotaryHalfSplit(Part):
 
     def load(self, tensors, rt):
         inv_freq = self.inv_freq()
+        self.rates = inv_freq.contiguous().to(rt.device)
+        if not self.tables:
+            return
         pos = torch.arange(self.max_positions, dtype=torch.float32)
         ang = pos[:, None] * inv_freq[None, :]
         self.cos = torch.cos(ang).contiguous().to(rt.device)
         self.sin = torch.sin(ang).contiguous().to(rt.device)
 
     def rotation(self):
+        if not self.tables:
+            return None
         return self.cos, self.sin, self.rotary_dims
+
+    def rotation_rates(self):
+        """(inv_freq float32 [rotary_dims / 2] on the GPU, rotary_dims): entry i turns by position * inv_freq[i]."""
+        return self.rates, self.rotary_dims

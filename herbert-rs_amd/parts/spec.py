@@ -20,7 +20,7 @@ class LayerSpec:
     """One layer: how its parts are arranged (`block`) and which parts they are."""
     block: PartSpec            # the arrangement, e.g. "prenorm"
     mixer: PartSpec
-    feed_forward: PartSpec
+    feed_forward: Optional[PartSpec]      # None: the layer has none (the block must allow that)
     norms: Dict[str, PartSpec]  # by the role the block gives them, e.g. "input", "post_mixer"
 
 
