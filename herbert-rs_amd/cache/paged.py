@@ -179,12 +179,14 @@ class Cache:
                 for e in entries:
                     self._kv_of[e] = group
             elif isinstance(need, StateNeed):
-                group = StateGroup(need, entries, self.n_slots, device)
-                self.state_groups[need] = group
-                for e in entries:
-                    self._state_of.setdefault(e, []).append(group)
+                self.state_groups[need] = StateGroup(need, entries, self.n_slots, device)
             else:
                 raise CacheError(f"unknown cache need {need!r}")
+        # an entry's states in the order in which its mixer names them, whichever groups they fell into
+        for entry, need in needs.items():
+            for one in (need if isinstance(need, (tuple, list)) else (need,)):
+                if isinstance(one, StateNeed):
+                    self._state_of.setdefault(entry, []).append(self.state_groups[one])
 
     @staticmethod
     def bytes_needed(needs, max_tokens, dtype, max_slots=None):

@@ -26,6 +26,9 @@ from .batch import StepEntry
 from .engine import Engine
 
 
+PARTIAL_PAGES = 64
+
+
 class Replayer:
     def __init__(self, engine, out_dir):
         self.engine = engine
@@ -65,10 +68,12 @@ def main(argv=None):
     ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
     ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
     ap.add_argument("--max-tokens", type=int, required=True,
-                    help="most tokens live requests hold at any time (each rounded up to 64)")
+                    help="most tokens live requests hold at any time")
     args = ap.parse_args(argv)
     try:
-        engine = Engine.from_folder(args.model, dtype=args.dtype, max_tokens=args.max_tokens)
+        # the pages hold 64 positions each and a request's last page is rarely full: room for the
+        # unused ends of the pages of up to PARTIAL_PAGES requests at a time beside the tokens themselves
+        engine = Engine.from_folder(args.model, dtype=args.dtype, max_tokens=args.max_tokens + 64 * PARTIAL_PAGES)
         replayer = Replayer(engine, args.out)
         for number, line in enumerate(sys.stdin, 1):
             line = line.strip()
