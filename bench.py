@@ -137,6 +137,90 @@ def run_workload(args, index, new=None):
     }
 
 
+# ---- the family with recurrent, latent-attention and routed layers, beside the dense decoder at equal size
+FAMILY_SIZES = {
+    # name: (width, layers, heads, key dim, value dim, latent rank, rotated part, experts, top, expert ff, vocab)
+    "small": (1024, 4, 8, 128, 128, 256, 64, 16, 2, 512, 32768),
+    "medium": (2048, 8, 16, 128, 128, 512, 64, 32, 4, 768, 32768),
+    "wide": (4096, 4, 32, 128, 128, 512, 64, 64, 4, 1536, 32768),
+}
+
+
+def family_configs(size):
+    """(Vipalorn config dict, Qwen3 config dict) of one size: three recurrent layers to one attention
+    layer, and the dense decoder with the same width, depth and heads, whose feed-forward is as wide as
+    the experts that a token uses together."""
+    W, L, H, D, V, rank, rot, E, top, ff, vocab = FAMILY_SIZES[size]
+    delta = {"type": "delta", "mixer": {"heads": H, "kv_heads": H // 2, "dim": D, "vdim": V, "conv": 4}}
+    latent = {"type": "latent_attention", "mixer": {"heads": H, "dim": D, "rot_dim": rot, "vdim": V, "kv_rank": rank,
+                                                    "scale": (D + rot) ** -0.5, "rot": {"base": 10000.0, "dims": rot}}}
+    mlp = {"kind": "moe", "expert": {"ff": ff, "limit": 7.0}, "router": {"experts": E, "top": top}}
+    layers = [dict(latent if i % 4 == 3 else delta, mlp=mlp) for i in range(L)]
+    vip = {"architecture": "Vipalorn", "vocab": vocab, "width": W, "layers": layers, "norm": {"eps": 1e-5},
+           "residual_mult": 0.5, "logit_scale": 1.0}
+    dense = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=L, hidden_size=W,
+                 num_attention_heads=H, num_key_value_heads=H // 2, head_dim=D, intermediate_size=top * ff,
+                 vocab_size=vocab, rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=True,
+                 max_position_embeddings=8192, eos_token_id=1)
+    return vip, dense
+
+
+def run_family(args):
+    """Prompt and decode throughput of the Vipalorn design at one size (random weights), beside the dense
+    Qwen3 decoder at equal size, both through the generation loop: prompts of 512 and 2,048 tokens alone,
+    and batches of 1, 8 and 32 sequences of 1,024 prompt tokens decoding `--steps` tokens each."""
+    import torch
+    import herbert_rs_amd as hb
+    from herbert_rs_amd.config.registry import resolve_architecture
+    from herbert_rs_amd.sampling import SamplingParams
+    torch.cuda.set_device(0)
+    new = max(args.steps, 8)
+    out = {}
+    for name, raw in zip(("vipalorn", "qwen3"), family_configs(args.size)):
+        arch = resolve_architecture(raw)
+        cfg = arch.config_class.from_dict(raw)
+        t0 = time.time()
+        engine = hb.Engine.from_config(cfg, architecture=arch, seed=7, dtype=args.dtype, max_tokens=32 * (1024 + new + 128),
+                                       max_slots=32)
+        print(f"[bench] {name} ({args.size}) built in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
+        gen = torch.Generator().manual_seed(3)
+        vocab = cfg.vocab_size
+
+        def ids(n):
+            return torch.randint(0, vocab, (n,), generator=gen).tolist()
+        quick = SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True, repeat_check=False)
+        rec = {}
+        for n in (512, 2048):
+            engine.generate([ids(n)], quick)
+            reps, t = 3, 0.0
+            for _ in range(reps):
+                engine.generate([ids(n)], quick)
+                t += engine.last_generation_stats.prefill_seconds
+            rec[f"prefill_{n}_tok_s"] = round(n * reps / t, 1)
+        for batch in (1, 8, 32):
+            prompts = [ids(1024) for _ in range(batch)]
+            params = SamplingParams(temperature=0.0, max_tokens=new, ignore_eos=True, repeat_check=False)
+            engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=4, ignore_eos=True, repeat_check=False),
+                            max_batch=batch)
+            engine.generate(prompts, params, max_batch=batch)
+            st = engine.last_generation_stats
+            rec[f"decode_b{batch}_tok_s"] = round((st.generated_tokens - batch) / st.decode_seconds, 1)
+            rec[f"decode_b{batch}_ms"] = round(st.decode_seconds / st.decode_steps * 1e3, 4)
+        out[name] = rec
+        print(f"[bench] {name}: {rec}", file=sys.stderr, flush=True)
+        del engine
+        torch.cuda.empty_cache()
+    v = out["vipalorn"]
+    return {"metric": f"decode tok/s, Vipalorn design ({args.size} sizes), batch 8, 1024 prompt tokens", "value": v["decode_b8_tok_s"],
+            "unit": "tokens/s", "n_gpus": 1, "steps": new, "warmup": 4, "ms_per_step": v["decode_b8_ms"],
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic: random weights, random token ids",
+            "config": {"model": f"Vipalorn {args.size}", "sizes": dict(zip(
+                ("width", "layers", "heads", "key_dim", "value_dim", "latent_rank", "rotated", "experts", "top", "expert_ff", "vocab"),
+                FAMILY_SIZES[args.size])), "global_batch": 8, "parallelism": "single GPU"},
+            "vipalorn": v, "qwen3_equal_size": out["qwen3"]}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -152,7 +236,8 @@ def main():
     ap.add_argument("--no-sweep", action="store_true", help="time the full context only, not 512 and the mean")
     ap.add_argument("--no-long", action="store_true",
                     help="skip the further sizes and lengths (contexts of 16 K and 32 K, batch 128 and 256, long prompts)")
-    ap.add_argument("--workload", default="headline", choices=["headline", "qwen3-1.7b", "qwen3-32b"],
+    ap.add_argument("--size", default="medium", choices=sorted(FAMILY_SIZES), help="layer sizes of --workload vipalorn")
+    ap.add_argument("--workload", default="headline", choices=["headline", "qwen3-1.7b", "qwen3-32b", "vipalorn"],
                     help="headline: BASELINE.json configs[2]; the others: configs[3] and configs[4]")
     ap.add_argument("--prefill-tokens", type=int, default=2048, help="length of the prompt of the prefill figure")
     ap.add_argument("--prefill-chunk", type=int, default=0,
@@ -171,6 +256,9 @@ def main():
               "does no work on several GPUs)")
         return 2
 
+    if args.workload == "vipalorn":
+        print(json.dumps(run_family(args)))
+        return 0
     if args.workload != "headline":
         print(json.dumps(run_workload(args, 3 if args.workload == "qwen3-1.7b" else 4,
                                       new=None if args.steps == 32 else args.steps)))

@@ -35,7 +35,7 @@ __device__ __forceinline__ void rotate_pair(float a, float b, float angle, float
 template <class TC>
 __global__ void latent_write_kernel(const float* __restrict__ down, int down_ld, const float* __restrict__ norm_w,
                                     const float* __restrict__ q, int q_ld, float* __restrict__ q_full,
-                                    const float* __restrict__ inv_freq, const int* __restrict__ positions,
+                                    bf16* __restrict__ q_plain, const float* __restrict__ inv_freq, const int* __restrict__ positions,
                                     const int* __restrict__ seq_of, const int* __restrict__ slots,
                                     const int* __restrict__ page_table, int max_pages, int page_size,
                                     TC* __restrict__ pages, int H, int qd, int rank, int rot, int rot_dims,
@@ -78,21 +78,27 @@ __global__ void latent_write_kernel(const float* __restrict__ down, int down_ld,
         }
         q_full[((size_t)t * H + h) * (rank + rot) + rank + i] = v;
     }
+    // the unrotated parts once more as bfloat16 [T, H, qd], for a matrix-core product with W_uk^T
+    if (q_plain)
+        for (int e = threadIdx.x; e < H * qd; e += blockDim.x) {
+            const int h = e / qd, i = e % qd;
+            q_plain[(size_t)t * H * qd + e] = hb_from_float<bf16>(q[(size_t)t * q_ld + (size_t)h * (qd + rot) + i]);
+        }
 }
 
 extern "C" int hb_latent_write(const float* down, int down_ld, const float* norm_w, const float* q, int q_ld, float* q_full,
-                               const float* inv_freq, const int* positions, const int* seq_of, const int* slots,
+                               void* q_plain, const float* inv_freq, const int* positions, const int* seq_of, const int* slots,
                                const int* page_table, int max_pages, int page_size, void* pages, int dtype, int T,
                                int H, int qd, int rank, int rot, int rot_dims, float eps, int write_cache,
                                hipStream_t stream) {
     HB_REQUIRE(T > 0 && H > 0 && rank > 0 && rot >= 0 && qd >= 0, "latent write: empty input");
     HB_REQUIRE(rot_dims >= 0 && rot_dims <= rot && rot_dims % 2 == 0, "latent write: %d rotated of %d", rot_dims, rot);
     if (dtype == HB_F32)
-        latent_write_kernel<float><<<T, 256, 0, stream>>>(down, down_ld, norm_w, q, q_ld, q_full, inv_freq, positions, seq_of, slots,
+        latent_write_kernel<float><<<T, 256, 0, stream>>>(down, down_ld, norm_w, q, q_ld, q_full, (bf16*)q_plain, inv_freq, positions, seq_of, slots,
                                                           page_table, max_pages, page_size, (float*)pages, H, qd,
                                                           rank, rot, rot_dims, eps, write_cache);
     else if (dtype == HB_BF16)
-        latent_write_kernel<bf16><<<T, 256, 0, stream>>>(down, down_ld, norm_w, q, q_ld, q_full, inv_freq, positions, seq_of, slots,
+        latent_write_kernel<bf16><<<T, 256, 0, stream>>>(down, down_ld, norm_w, q, q_ld, q_full, (bf16*)q_plain, inv_freq, positions, seq_of, slots,
                                                          page_table, max_pages, page_size, (bf16*)pages, H, qd,
                                                          rank, rot, rot_dims, eps, write_cache);
     else

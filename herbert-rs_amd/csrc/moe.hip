@@ -282,3 +282,148 @@ extern "C" int hb_moe_combine(const float* y, const float* weight, const int* ro
     HB_CHECK_LAUNCH("moe_combine");
     return 0;
 }
+
+// ------------------------------------------------------------------------ products on the matrix cores
+// The same products for bfloat16 operands with float32 sums (v_mfma_f32_16x16x32_bf16), and more
+// generally a group of products that share a shape: group g multiplies rows of A (from column
+// g * a_group_off on) with its own matrix W[g] [N, K] into columns of C from g * c_group_off on.
+// The rows of a group come as a list of tiles (group, first row, rows <= 64) or, without a list, as
+// every group's ceil(M / 64) tiles of the same M rows (heads that each have a matrix of their own).
+// A workgroup is four waves on one tile of 64 rows; a wave holds two blocks of 16 weight rows
+// against up to four blocks of 16 activation rows (the blocks beyond the tile's rows are skipped, so
+// a tile of a few rows costs little more than streaming its weights). Operands go from memory
+// straight into the lanes: lane l of an operand holds 8 consecutive k of row l % 16 from k0 + 8 (l / 16).
+// An output is summed over k in the same order whatever else the tile holds.
+// EPI 0: float32 C. EPI 1: bfloat16 C. EPI 2: W[g] is [2 F, K], gate rows then up rows; a wave's two
+// blocks are 16 gate rows and the 16 up rows that go with them, and C [*, F] bfloat16 receives
+// min(gate, limit) sigmoid(alpha min(gate, limit)) (clamp(up, -limit, limit) + 1).
+typedef __bf16 hb_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float hb_f32x4 __attribute__((ext_vector_type(4)));
+
+template <int EPI>
+__global__ void __launch_bounds__(256)
+grouped_mfma_kernel(const bf16* __restrict__ A, int lda, size_t a_group_off, const bf16* __restrict__ W, int N,
+                    int K, void* __restrict__ Cv, int ldc, size_t c_group_off, const int* __restrict__ order,
+                    int top, const int* __restrict__ tile_group, const int* __restrict__ tile_row0,
+                    const int* __restrict__ tile_rows, int M, int m_tiles, float limit, float alpha) {
+    int group, row0, rows;
+    if (tile_group) {
+        group = tile_group[blockIdx.y];
+        if (group < 0) return;
+        row0 = tile_row0[blockIdx.y];
+        rows = tile_rows[blockIdx.y];
+    } else {
+        group = blockIdx.y / m_tiles;
+        row0 = (blockIdx.y % m_tiles) * MOE_TILE_M;
+        rows = M - row0 < MOE_TILE_M ? M - row0 : MOE_TILE_M;
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r16 = lane & 15, g4 = lane >> 4;
+    const int F = N / 2;
+    const int out_cols = EPI == 2 ? F : N;
+    // the first of the wave's output columns; its weight rows: [n0, n0 + 32), or with EPI 2 [n0, + 16) and [F + n0, + 16)
+    const int n0 = EPI == 2 ? (blockIdx.x * 4 + wave) * 16 : (blockIdx.x * 4 + wave) * 32;
+    if (n0 >= out_cols) return;
+    const bf16* Wg = W + (size_t)group * N * K;
+    const bf16* wrow[2];
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+        int n = (EPI == 2 ? (a == 0 ? n0 : F + n0) : n0 + 16 * a) + r16;
+        if (n >= N) n = N - 1;                       // (read a row that exists; its sums are not stored)
+        wrow[a] = Wg + (size_t)n * K + g4 * 8;
+    }
+    const int blocks = (rows + 15) / 16;
+    const bf16* xrow[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        int m = b * 16 + r16;
+        if (m >= rows) m = rows - 1;
+        const int src = top > 0 ? order[row0 + m] / top : row0 + m;
+        xrow[b] = A + (size_t)src * lda + (size_t)group * a_group_off + g4 * 8;
+    }
+    hb_f32x4 acc[2][4];
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) acc[a][b] = hb_f32x4{0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll 4
+    for (int k = 0; k < K; k += 32) {
+        hb_bf16x8 wv[2], xv[4];
+#pragma unroll
+        for (int a = 0; a < 2; ++a) wv[a] = *(const hb_bf16x8*)(wrow[a] + k);
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+            if (b < blocks) xv[b] = *(const hb_bf16x8*)(xrow[b] + k);
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+            if (b < blocks) {
+#pragma unroll
+                for (int a = 0; a < 2; ++a)
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[a], xv[b], acc[a][b], 0, 0, 0);
+            }
+    }
+    // lane: activation row b * 16 + r16, weight rows g4 * 4 + i of each block
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        const int m = b * 16 + r16;
+        if (b >= blocks || m >= rows) continue;
+        const size_t base = (size_t)(row0 + m) * ldc + (size_t)group * c_group_off;
+        if (EPI == 2) {
+            bf16* C = (bf16*)Cv;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int n = n0 + g4 * 4 + i;
+                if (n >= F) continue;
+                const float g = fminf(acc[0][b][i], limit);
+                const float u = fminf(fmaxf(acc[1][b][i], -limit), limit);
+                C[base + n] = hb_from_float<bf16>(g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+            }
+        } else {
+#pragma unroll
+            for (int a = 0; a < 2; ++a)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int n = n0 + 16 * a + g4 * 4 + i;
+                    if (n >= N) continue;
+                    if (EPI == 0)
+                        ((float*)Cv)[base + n] = acc[a][b][i];
+                    else
+                        ((bf16*)Cv)[base + n] = hb_from_float<bf16>(acc[a][b][i]);
+                }
+        }
+    }
+}
+
+// tile_group null: `groups` groups of ceil(M / 64) tiles each over the same M rows; else a list of
+// n_tiles tiles (a group < 0 ends a tile at once). K in steps of 32; lda, a_group_off and the matrices
+// such that every operand's 8 numbers lie at a multiple of 16 bytes.
+extern "C" int hb_grouped_mfma(const void* A, int lda, size_t a_group_off, const void* W, int N, int K, void* C,
+                               int ldc, size_t c_group_off, int epi, const int* order, int top,
+                               const int* tile_group, const int* tile_row0, const int* tile_rows, int n_tiles, int M,
+                               int groups, float limit, float alpha, hipStream_t stream) {
+    HB_REQUIRE(N > 0 && K > 0 && K % 32 == 0, "grouped product: K = %d must be a positive multiple of 32", K);
+    HB_REQUIRE(lda % 8 == 0 && a_group_off % 8 == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0,
+               "grouped product: operands must lie at multiples of 16 bytes");
+    HB_REQUIRE(epi >= 0 && epi <= 2 && (epi != 2 || N % 2 == 0), "grouped product: unknown epilogue %d", epi);
+    int m_tiles = 0, tiles = n_tiles;
+    if (!tile_group) {
+        HB_REQUIRE(M > 0 && groups > 0 && top == 0, "grouped product: empty batch");
+        m_tiles = (M + MOE_TILE_M - 1) / MOE_TILE_M;
+        tiles = m_tiles * groups;
+    }
+    HB_REQUIRE(tiles > 0 && tiles <= 65535, "grouped product: %d row tiles exceed the grid", tiles);
+    const int out_cols = epi == 2 ? N / 2 : N;
+    const int per_group = epi == 2 ? 64 : 128;
+    const dim3 grid((out_cols + per_group - 1) / per_group, tiles);
+#define HB_GROUPED(E)                                                                                               \
+    grouped_mfma_kernel<E><<<grid, 256, 0, stream>>>((const bf16*)A, lda, a_group_off, (const bf16*)W, N, K, C, ldc, \
+                                                     c_group_off, order, top, tile_group, tile_row0, tile_rows, M,   \
+                                                     m_tiles, limit, alpha)
+    if (epi == 0) HB_GROUPED(0);
+    else if (epi == 1) HB_GROUPED(1);
+    else HB_GROUPED(2);
+#undef HB_GROUPED
+    HB_CHECK_LAUNCH("grouped_mfma");
+    return 0;
+}

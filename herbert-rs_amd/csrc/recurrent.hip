@@ -98,83 +98,105 @@ extern "C" int hb_conv_silu(const float* proj, int ld, const float* taps, float*
 // State S [D, V] a (slot, head). For every token of the sequence, in order:
 //   S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q        (o sees the token's own write)
 // with g = exp(-exp(A_log[h]) * softplus(a + dt_bias[h])) and beta = sigmoid(b), a and b columns of
-// the projection's row. The columns of S never meet: a lane owns one (D registers), a wave 64 of
-// them, and the wave walks the sequence's tokens. k and q of a token are the same for all lanes:
-// lane d holds element d (+ 64, + 128 ...) and the others read it from there.
+// the projection's row. The columns of S never meet, and the tokens are a chain: the kernel is as
+// fast as one token's step is short. A column is held by LPC lanes (each 32 of its D numbers, in
+// registers; LPC = 1, 2, 4 or 8 for D up to 256), a wave holds 64 / LPC columns and walks the
+// sequence's tokens; the two dot products a token are summed over a column's lanes by LPC - 1
+// exchanges. The token ahead is loaded while the present one is worked on, and g and beta of a
+// token do not wait for the chain.
 // qkv rows: [kv_heads x D queries | kv_heads x D keys | heads x V values]; head h reads the
 // query and key of kv head h / (heads / kv_heads).
-template <int DMAX>
+#define DELTA_PER 32
+
+template <int LPC>
+__device__ __forceinline__ float delta_column_sum(float v) {
+#pragma unroll
+    for (int off = 1; off < LPC; off <<= 1) v += __shfl_xor(v, off, HB_WAVE);
+    return v;
+}
+
+template <int LPC>
 __global__ void __launch_bounds__(HB_WAVE)
 gated_delta_kernel(const float* __restrict__ qkv, int C, const float* __restrict__ proj, int ld, int b_off,
                    int a_off, const float* __restrict__ A_log, const float* __restrict__ dt_bias,
                    float* __restrict__ state, const int* __restrict__ seq_starts, const int* __restrict__ slots,
                    float* __restrict__ out, int kv_heads, int heads, int D, int V) {
-    constexpr int PER = DMAX / HB_WAVE > 0 ? DMAX / HB_WAVE : 1;      // elements of k (and q) a lane holds
+    constexpr int COLS = HB_WAVE / LPC;
     const int seq = blockIdx.x, h = blockIdx.y;
     const int lane = threadIdx.x;
-    const int col = blockIdx.z * HB_WAVE + lane;
+    const int part = lane % LPC;                       // which 32 of the column's D numbers
+    const int col = blockIdx.z * COLS + lane / LPC;
     const bool live = col < V;
+    const int d0 = part * DELTA_PER;
     const int kvh = h / (heads / kv_heads);
     const int first = seq_starts[seq], last = seq_starts[seq + 1];
     float* S_mem = state + ((size_t)slots[seq] * heads + h) * D * V + col;
-    float S[DMAX];
+    float S[DELTA_PER];
+    // (numbers beyond D are zeros and stay zeros: their k and q are loaded as zeros)
 #pragma unroll
-    for (int d = 0; d < DMAX; ++d) S[d] = (live && d < D) ? S_mem[(size_t)d * V] : 0.f;
+    for (int i = 0; i < DELTA_PER; ++i) S[i] = (live && d0 + i < D) ? S_mem[(size_t)(d0 + i) * V] : 0.f;
     const float rate = -expf(A_log[h]);
     const float bias = dt_bias[h];
-    const int q_at = kvh * D, k_at = (kv_heads + kvh) * D, v_at = 2 * kv_heads * D + h * V;
+    const int q_at = kvh * D + d0, k_at = (kv_heads + kvh) * D + d0, v_at = 2 * kv_heads * D + h * V;
+    const bool whole = d0 + DELTA_PER <= D && (D % 4) == 0 && (C % 4) == 0;      // 16-byte loads of this lane's 32
 
-    // the token ahead is loaded while the present one is worked on
-    float kq[PER], qq[PER], vv = 0.f, aa = 0.f, bb = 0.f;
-    auto load = [&](int t, float* k_, float* q_, float& v_, float& a_, float& b_) {
+    float kn[DELTA_PER], qn[DELTA_PER], vn = 0.f, an = 0.f, bn = 0.f;
+    auto load = [&](int t) {
         const float* row = qkv + (size_t)t * C;
+        if (whole) {
 #pragma unroll
-        for (int i = 0; i < PER; ++i) {
-            const int d = lane + HB_WAVE * i;
-            k_[i] = d < D ? row[k_at + d] : 0.f;
-            q_[i] = d < D ? row[q_at + d] : 0.f;
-        }
-        v_ = live ? row[v_at + col] : 0.f;
-        a_ = proj[(size_t)t * ld + a_off + h];
-        b_ = proj[(size_t)t * ld + b_off + h];
-    };
-    if (first < last) load(first, kq, qq, vv, aa, bb);
-    for (int t = first; t < last; ++t) {
-        float kc[PER], qc[PER];
+            for (int i = 0; i < DELTA_PER; i += 4) {
+                const float4 kk = *(const float4*)(row + k_at + i);
+                const float4 qq = *(const float4*)(row + q_at + i);
+                kn[i] = kk.x, kn[i + 1] = kk.y, kn[i + 2] = kk.z, kn[i + 3] = kk.w;
+                qn[i] = qq.x, qn[i + 1] = qq.y, qn[i + 2] = qq.z, qn[i + 3] = qq.w;
+            }
+        } else {
 #pragma unroll
-        for (int i = 0; i < PER; ++i) {
-            kc[i] = kq[i];
-            qc[i] = qq[i];
-        }
-        const float vc = vv, ac = aa, bc = bb;
-        if (t + 1 < last) load(t + 1, kq, qq, vv, aa, bb);
-        const float z = ac + bias;
-        const float softplus = z > 20.f ? z : log1pf(expf(z));
-        const float g = expf(rate * softplus);
-        const float beta = 1.0f / (1.0f + expf(-bc));
-        float dot = 0.f;
-#pragma unroll
-        for (int d = 0; d < DMAX; ++d) {
-            if (d < D) {
-                S[d] *= g;
-                dot = fmaf(S[d], __shfl(kc[d / HB_WAVE], d % HB_WAVE, HB_WAVE), dot);
+            for (int i = 0; i < DELTA_PER; ++i) {
+                kn[i] = d0 + i < D ? row[k_at + i] : 0.f;
+                qn[i] = d0 + i < D ? row[q_at + i] : 0.f;
             }
         }
+        vn = live ? row[v_at + col] : 0.f;
+        an = proj[(size_t)t * ld + a_off + h];
+        bn = proj[(size_t)t * ld + b_off + h];
+    };
+    if (first < last) load(first);
+    for (int t = first; t < last; ++t) {
+        float kc[DELTA_PER], qc[DELTA_PER];
+#pragma unroll
+        for (int i = 0; i < DELTA_PER; ++i) {
+            kc[i] = kn[i];
+            qc[i] = qn[i];
+        }
+        const float vc = vn;
+        const float z = an + bias;
+        const float softplus = z > 20.f ? z : log1pf(expf(z));
+        const float g = expf(rate * softplus);
+        const float beta = 1.0f / (1.0f + expf(-bn));
+        if (t + 1 < last) load(t + 1);
+        float dot = 0.f;
+#pragma unroll
+        for (int i = 0; i < DELTA_PER; ++i) {
+            S[i] *= g;
+            dot = fmaf(S[i], kc[i], dot);
+        }
+        dot = delta_column_sum<LPC>(dot);
         const float u = beta * (vc - dot);
         float o = 0.f;
 #pragma unroll
-        for (int d = 0; d < DMAX; ++d) {
-            if (d < D) {
-                S[d] = fmaf(__shfl(kc[d / HB_WAVE], d % HB_WAVE, HB_WAVE), u, S[d]);
-                o = fmaf(S[d], __shfl(qc[d / HB_WAVE], d % HB_WAVE, HB_WAVE), o);
-            }
+        for (int i = 0; i < DELTA_PER; ++i) {
+            S[i] = fmaf(kc[i], u, S[i]);
+            o = fmaf(S[i], qc[i], o);
         }
-        if (live) out[(size_t)t * heads * V + h * V + col] = o;
+        o = delta_column_sum<LPC>(o);
+        if (live && part == 0) out[(size_t)t * heads * V + h * V + col] = o;
     }
     if (live) {
 #pragma unroll
-        for (int d = 0; d < DMAX; ++d)
-            if (d < D) S_mem[(size_t)d * V] = S[d];
+        for (int i = 0; i < DELTA_PER; ++i)
+            if (d0 + i < D) S_mem[(size_t)(d0 + i) * V] = S[i];
     }
 }
 
@@ -186,15 +208,16 @@ extern "C" int hb_gated_delta(const float* qkv, int C, const float* proj, int ld
     HB_REQUIRE(D > 0 && D <= 256, "delta rule: keys of %d, the kernel takes 1 to 256", D);
     HB_REQUIRE(V > 0 && C == 2 * kv_heads * D + heads * V, "delta rule: %d channels do not fit the heads", C);
     HB_REQUIRE(B <= 65535 && heads <= 65535, "delta rule: too many sequences or heads for the grid");
-    const dim3 grid(B, heads, (V + HB_WAVE - 1) / HB_WAVE);
-#define HB_DELTA(DM)                                                                                              \
-    gated_delta_kernel<DM><<<grid, HB_WAVE, 0, stream>>>(qkv, C, proj, ld, b_off, a_off, A_log, dt_bias, state,   \
-                                                         seq_starts, slots, out, kv_heads, heads, D, V)
-    if (D <= 16) HB_DELTA(16);
-    else if (D <= 32) HB_DELTA(32);
-    else if (D <= 64) HB_DELTA(64);
-    else if (D <= 128) HB_DELTA(128);
-    else HB_DELTA(256);
+    const int lpc = D <= 32 ? 1 : D <= 64 ? 2 : D <= 128 ? 4 : 8;
+    const int cols = HB_WAVE / lpc;
+    const dim3 grid(B, heads, (V + cols - 1) / cols);
+#define HB_DELTA(L)                                                                                               \
+    gated_delta_kernel<L><<<grid, HB_WAVE, 0, stream>>>(qkv, C, proj, ld, b_off, a_off, A_log, dt_bias, state,     \
+                                                        seq_starts, slots, out, kv_heads, heads, D, V)
+    if (lpc == 1) HB_DELTA(1);
+    else if (lpc == 2) HB_DELTA(2);
+    else if (lpc == 4) HB_DELTA(4);
+    else HB_DELTA(8);
 #undef HB_DELTA
     HB_CHECK_LAUNCH("gated_delta");
     return 0;

@@ -19,10 +19,11 @@ def _check_pages(meta, cache, T, width):
 
 
 def latent_write(proj, q_off, down_off, norm_w, q_full, inv_freq, meta, cache, H, qd, rank, rot, rot_dims, eps,
-                 write_cache=True):
+                 write_cache=True, q_plain=None):
     """proj f32 [T, ld]: columns [down_off, + rank + rot) -> the tokens' cache rows (the latent RMS-normed
     with norm_w, the rest rotated); columns [q_off, + H (qd + rot)) are the queries, whose rotated parts
-    go into q_full f32 [T, H (rank + rot)]."""
+    go into q_full f32 [T, H (rank + rot)] and, if q_plain (bf16 [T, H qd]) is given, whose unrotated
+    parts are copied there."""
     T, ld = proj.shape
     _check(proj, "proj", torch.float32, (T, ld))
     if min(q_off, down_off) < 0 or q_off + H * (qd + rot) > ld or down_off + rank + rot > ld:
@@ -34,9 +35,11 @@ def latent_write(proj, q_off, down_off, norm_w, q_full, inv_freq, meta, cache, H
     if rot_dims % 2 or not 0 <= rot_dims <= rot:
         raise BackendError(f"latent write: {rot_dims} rotated entries of {rot}")
     _check_pages(meta, cache, T, rank + rot)
+    if q_plain is not None:
+        _check(q_plain, "q_plain", torch.bfloat16, (T, H * qd))
     base = proj.data_ptr()
     lib.call("attention_latent", "hb_latent_write", base + 4 * down_off, ld, norm_w.data_ptr(), base + 4 * q_off, ld,
-             q_full.data_ptr(), _ptr(inv_freq), meta.positions.data_ptr(), meta.seq_of.data_ptr(),
+             q_full.data_ptr(), _ptr(q_plain), _ptr(inv_freq), meta.positions.data_ptr(), meta.seq_of.data_ptr(),
              meta.slots.data_ptr(), cache.page_table.data_ptr(), cache.page_table.shape[1], cache.page_size,
              cache.k.data_ptr(), dtype_code(cache.k), T, H, qd, rank, rot, rot_dims, float(eps),
              1 if write_cache else 0, _stream())

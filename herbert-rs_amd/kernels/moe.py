@@ -87,3 +87,42 @@ def combine(y, routing, x):
     _check(x, "x", torch.float32, (r.T, H))
     lib.call("moe", "hb_moe_combine", y.data_ptr(), r.weight.data_ptr(), r.row_of.data_ptr(), x.data_ptr(), r.T,
              r.top, H, _stream())
+
+
+EPI_F32, EPI_BF16, EPI_GLU = 0, 1, 2
+
+
+def mfma_takes(K, lda, a_group_off=0):
+    """True if the matrix-core kernel takes products of this inner size and layout (bfloat16 operands)."""
+    return K % 32 == 0 and lda % 8 == 0 and a_group_off % 8 == 0
+
+
+def grouped_mfma(a, lda, a_group_off, w, c, ldc, c_group_off, epi, routing=None, gather=False, M=0, limit=0.0,
+                 alpha=0.0):
+    """Group g: C[rows, g * c_group_off + n] = sum_k A[src(row), g * a_group_off + k] * w[g][n, k], bfloat16
+    operands, float32 sums. With `routing` the rows are the (token, expert) pairs in their experts' order
+    (gather: A's rows are the tokens'); without, every group takes the same M rows. epi: EPI_F32 / EPI_BF16
+    store C in that type; EPI_GLU: w[g] is [2 F, K] (gate rows, then up rows) and C bfloat16 [*, F] receives
+    the experts' activation with `limit` and `alpha`."""
+    G, N, K = w.shape
+    _check(a, "a", torch.bfloat16)
+    _check(w, "w", torch.bfloat16, (G, N, K))
+    _check(c, "c", torch.bfloat16 if epi != EPI_F32 else torch.float32)
+    if not mfma_takes(K, lda, a_group_off):
+        raise BackendError(f"grouped product: K = {K}, rows {lda} apart and groups {a_group_off} apart are not taken")
+    out_cols = N // 2 if epi == EPI_GLU else N
+    if routing is not None:
+        r = routing
+        rows_a, rows_c = (r.T if gather else r.T * r.top), r.T * r.top
+        if G != r.E:
+            raise BackendError("grouped product: one matrix an expert")
+        lists = (r.order.data_ptr(), r.top if gather else 0, r.tile_expert.data_ptr(), r.tile_row0.data_ptr(),
+                 r.tile_rows.data_ptr(), r.tiles, 0, 0)
+    else:
+        rows_a = rows_c = M
+        lists = (None, 0, None, None, None, 0, M, G)
+    if (rows_a - 1) * lda + (G - 1) * a_group_off + K > a.numel() or \
+            (rows_c - 1) * ldc + (G - 1) * c_group_off + out_cols > c.numel():
+        raise BackendError("grouped product: an operand does not hold every row that is addressed")
+    lib.call("moe", "hb_grouped_mfma", a.data_ptr(), lda, a_group_off, w.data_ptr(), N, K, c.data_ptr(), ldc,
+             c_group_off, epi, *lists, float(limit), float(alpha), _stream())

@@ -15,7 +15,7 @@ Scores, softmax and the weighted sums are float32 in either mode.
 import torch
 
 from ..cache import KVNeed
-from ..kernels import latent, ops
+from ..kernels import latent, moe, ops
 from ..weights import TensorNeed
 from .base import Part
 from .linear import Linear
@@ -82,17 +82,27 @@ class LatentAttention(Part):
         proj = rt.buffer("latent_proj", (T, self.width), torch.float32)
         self.proj.forward(y, proj)
         q_full = rt.buffer("latent_q_full", (T, H * self.row), torch.float32)
+        cores = rt.dtype == torch.bfloat16 and moe.mfma_takes(self.dim, H * self.dim, self.dim) \
+            and moe.mfma_takes(self.rank, H * self.rank, self.rank)
+        q_plain = rt.buffer("latent_q_plain", (T, H * self.dim), torch.bfloat16) if cores else None
         latent.latent_write(proj, 0, self.q_width, self.norm_w, q_full, self.inv_freq, ctx.meta, kv, H, self.dim,
-                            self.rank, self.rot_dim, self.rot_dims, self.eps, write_cache=ctx.owns_cache)
-        # q'[t, n, :] = W_uk,n^T q[t, n, :dim]: a product a head, all in one launch
-        ops.gemm_plain_batched(proj, self.uk_t, q_full, T, self.rank, self.dim, self.width, self.dim,
-                               H * self.row, H, self.dim + self.rot_dim, self.rank * self.dim, self.row)
+                            self.rank, self.rot_dim, self.rot_dims, self.eps, write_cache=ctx.owns_cache,
+                            q_plain=q_plain)
+        # q'[t, n, :] = W_uk,n^T q[t, n, :dim]: a product a head, all heads in one launch
+        if cores:
+            moe.grouped_mfma(q_plain, H * self.dim, self.dim, self.uk_t, q_full, H * self.row, self.row, moe.EPI_F32, M=T)
+        else:
+            ops.gemm_plain_batched(proj, self.uk_t, q_full, T, self.rank, self.dim, self.width, self.dim,
+                                   H * self.row, H, self.dim + self.rot_dim, self.rank * self.dim, self.row)
         mixed = rt.buffer("latent_mixed", (T, H * self.rank))
         latent.latent_attention_plain(q_full, ctx.meta, kv, mixed, proj if self.gated else None,
                                       self.q_width + self.row, H, self.rank, self.rot_dim, self.scale)
         # a head's summed latents through its W_uv
         attn = rt.buffer("latent_attn", (T, H * self.vdim))
-        ops.gemm_plain_batched(mixed, self.uv, attn, T, self.vdim, self.rank, H * self.rank, self.rank, H * self.vdim,
-                               H, self.rank, self.vdim * self.rank, self.vdim)
+        if cores:
+            moe.grouped_mfma(mixed, H * self.rank, self.rank, self.uv, attn, H * self.vdim, self.vdim, moe.EPI_BF16, M=T)
+        else:
+            ops.gemm_plain_batched(mixed, self.uv, attn, T, self.vdim, self.rank, H * self.rank, self.rank,
+                                   H * self.vdim, H, self.rank, self.vdim * self.rank, self.vdim)
         left = ctx.leave_norm(self.o, x)
         self.o.forward(attn, x, accumulate=True, leave=None if left is None else left.leave())

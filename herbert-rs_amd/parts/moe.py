@@ -12,6 +12,7 @@ import torch
 from ..kernels import moe, ops
 from ..weights import TensorNeed
 from .base import Part
+from .linear import Linear
 from .registry import register
 
 GATE_ALPHA = 1.702
@@ -48,7 +49,7 @@ class RoutedExperts(Part):
 
     def load(self, tensors, rt):
         n = self.names
-        self.router = rt.weight(tensors[n["router"]])
+        self.router = Linear(rt.weight(tensors[n["router"]]), scratch=rt.scratch)
         self.router_bias = rt.weight(tensors[n["router_bias"]], matrix=False) if n.get("router_bias") else None
         # [E, 2 F, W]: an expert's gate rows, then its up rows; [E, W, F]
         self.gate_up = torch.stack([torch.cat([rt.weight(tensors[n["gate"].format(e=e)]),
@@ -60,14 +61,20 @@ class RoutedExperts(Part):
         rt = ctx.rt
         T, E, top, F = y.shape[0], self.experts, self.top, self.inter
         logits = rt.buffer("moe_logits", (T, E), torch.float32)
-        ops.gemm_plain(y, self.router, logits)
+        self.router.forward(y, logits)          # float32 sums of the rows' products with the router's matrix
         routing = moe.Routing(rt.buffer("moe_ints", (moe.Routing.ints_needed(T, E, top),), torch.int32),
                               rt.buffer("moe_weight", (T, top), torch.float32), T, E, top)
         moe.route(logits, self.router_bias, routing)
-        gu = rt.buffer("moe_gate_up", (T * top, 2 * F), torch.float32)
-        moe.gemm_plain(y, self.gate_up, gu, routing, gather=True)
         act = rt.buffer("moe_act", (T * top, F))
-        moe.activate(gu, act, self.limit, self.alpha)
         out = rt.buffer("moe_out", (T * top, self.hidden_size), torch.float32)
-        moe.gemm_plain(act, self.down, out, routing, gather=False)
+        if y.dtype == torch.bfloat16 and moe.mfma_takes(self.hidden_size, self.hidden_size) and moe.mfma_takes(F, F):
+            # matrix cores; the activation is the first product's epilogue
+            moe.grouped_mfma(y, self.hidden_size, 0, self.gate_up, act, F, 0, moe.EPI_GLU, routing, gather=True,
+                             limit=self.limit, alpha=self.alpha)
+            moe.grouped_mfma(act, F, 0, self.down, out, self.hidden_size, 0, moe.EPI_F32, routing)
+        else:
+            gu = rt.buffer("moe_gate_up", (T * top, 2 * F), torch.float32)
+            moe.gemm_plain(y, self.gate_up, gu, routing, gather=True)
+            moe.activate(gu, act, self.limit, self.alpha)
+            moe.gemm_plain(act, self.down, out, routing, gather=False)
         moe.combine(out, routing, x)
