@@ -200,3 +200,221 @@ extern "C" int hb_latent_attention_plain(const float* q_full, const void* pages,
     HB_CHECK_LAUNCH("latent_attention_plain");
     return 0;
 }
+
+// ------------------------------------------------ the same attention on the matrix cores (bfloat16 rows)
+// A wave takes 16 heads of one token (the rows of its matrix products) and a range of the keys, in
+// chunks of 32. Scores: S^T = K Q^T, the chunk's rows straight from memory as operands (a lane: one
+// key's 8 consecutive numbers), the query (times the scale) in registers as two bfloat16 halves, high
+// and low, so that it keeps 16 bits of mantissa. The sums are float32, and so are the softmax and its
+// state, which are a lane's own (a lane holds scores of one head only). Weighted sums: O^T = V^T P^T
+// with the weights again as high and low halves (they are never rounded to 8 bits), and V^T, the
+// chunk's first `rank` numbers a key with the keys along a row, transposed through LDS. The 32 keys
+// of a product stand in the order in which the scores' lanes hold them (4 g + i of the first block of
+// 16, then of the second), so the weights go from the scores' registers into the next product as they
+// are. With more than one range a token the unnormalised sums, maxima and denominators go to scratch
+// and a second kernel joins them in the ranges' order.
+// Sizes: rank a multiple of 16, rank + rot a multiple of 32; RB >= rank / 16, KSM >= (rank + rot) / 32.
+typedef __bf16 la_bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 la_bf16x4 __attribute__((ext_vector_type(4)));
+typedef float la_f32x4 __attribute__((ext_vector_type(4)));
+#define LA_CHUNK 32
+#define LA_VT_STRIDE 36          // bfloat16 a row of V^T in LDS: 32 keys and 8 bytes, so rows start at other banks
+
+__device__ __forceinline__ void la_split(float v, __bf16& hi, __bf16& lo) {
+    hi = (__bf16)v;
+    lo = (__bf16)(v - (float)hi);
+}
+
+template <int RB, int KSM>
+__global__ void __launch_bounds__(HB_WAVE)
+latent_attention_mfma_kernel(const float* __restrict__ q_full, const bf16* __restrict__ pages,
+                             bf16* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml,
+                             const float* __restrict__ gate, int gate_ld, const int* __restrict__ positions,
+                             const int* __restrict__ seq_of, const int* __restrict__ slots,
+                             const int* __restrict__ page_table, int max_pages, int page_size, int H, int rank,
+                             int rot, float scale, int splits, int chunks_per_split) {
+    __shared__ __attribute__((aligned(16))) __bf16 Vt[RB * 16 * LA_VT_STRIDE];
+    const int HB = (H + 15) / 16;
+    const int t = blockIdx.x / HB, hb = blockIdx.x % HB, split = blockIdx.y;
+    const int lane = threadIdx.x, n = lane & 15, g = lane >> 4;
+    const int h = hb * 16 + n;
+    const bool head = h < H;
+    const int pos = positions[t];
+    const int* pt = page_table + (size_t)slots[seq_of[t]] * max_pages;
+    const int kd = rank + rot, KS = kd / 32, rblocks = rank / 16;
+
+    la_bf16x8 qh[KSM], ql[KSM];
+    {
+        const float* qrow = q_full + ((size_t)t * H + (head ? h : H - 1)) * kd + 8 * g;
+#pragma unroll
+        for (int ks = 0; ks < KSM; ++ks)
+            if (ks < KS) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    __bf16 hi, lo;
+                    la_split(qrow[32 * ks + e] * scale, hi, lo);
+                    qh[ks][e] = hi;
+                    ql[ks][e] = lo;
+                }
+            }
+    }
+    const int n_chunks = (pos + LA_CHUNK) / LA_CHUNK;            // chunks that hold a key <= pos
+    const int c_begin = split * chunks_per_split;
+    const int c_end = n_chunks < c_begin + chunks_per_split ? n_chunks : c_begin + chunks_per_split;
+    float m = -INFINITY, l = 0.f;
+    la_f32x4 acc[RB];
+#pragma unroll
+    for (int db = 0; db < RB; ++db) acc[db] = la_f32x4{0.f, 0.f, 0.f, 0.f};
+
+    for (int c = c_begin; c < c_end; ++c) {
+        const int j0 = c * LA_CHUNK;
+        // the chunk's 32 keys lie in one page (pages hold a multiple of 32 positions)
+        const bf16* chunk = pages + ((size_t)pt[j0 / page_size] * page_size + j0 % page_size) * kd;
+        la_f32x4 s[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            s[kb] = la_f32x4{0.f, 0.f, 0.f, 0.f};
+            const bf16* krow = chunk + (size_t)(kb * 16 + n) * kd + 8 * g;
+#pragma unroll
+            for (int ks = 0; ks < KSM; ++ks)
+                if (ks < KS) {
+                    const la_bf16x8 kv = *(const la_bf16x8*)(krow + 32 * ks);
+                    s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kv, qh[ks], s[kb], 0, 0, 0);
+                    s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kv, ql[ks], s[kb], 0, 0, 0);
+                }
+        }
+        // s[kb][i]: key j0 + 16 kb + 4 g + i against head n
+        float cmax = -INFINITY;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (j0 + 16 * kb + 4 * g + i > pos) s[kb][i] = -INFINITY;
+                cmax = fmaxf(cmax, s[kb][i]);
+            }
+        cmax = fmaxf(cmax, __shfl_xor(cmax, 16, HB_WAVE));
+        cmax = fmaxf(cmax, __shfl_xor(cmax, 32, HB_WAVE));
+        const float m_new = fmaxf(m, cmax);                     // finite: the chunk holds a key <= pos
+        const float corr = expf(m - m_new);
+        la_bf16x8 ph, pl;
+        float psum = 0.f;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float p = expf(s[kb][i] - m_new);
+                psum += p;
+                __bf16 hi, lo;
+                la_split(p, hi, lo);
+                ph[4 * kb + i] = hi;
+                pl[4 * kb + i] = lo;
+            }
+        l = l * corr + psum;
+        m = m_new;
+#pragma unroll
+        for (int db = 0; db < RB; ++db)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[db][i] *= corr;
+        // V^T into LDS: lane: key lane % 32, 8 numbers of it at a time
+        {
+            const int kk = lane & 31;
+            const bf16* vrow = chunk + (size_t)kk * kd;
+            for (int c8 = lane >> 5; c8 < rank / 8; c8 += 2) {
+                const la_bf16x8 v = *(const la_bf16x8*)(vrow + 8 * c8);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) Vt[(8 * c8 + e) * LA_VT_STRIDE + kk] = v[e];
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int db = 0; db < RB; ++db)
+            if (db < rblocks) {
+                const __bf16* vr = Vt + (db * 16 + n) * LA_VT_STRIDE + 4 * g;
+                const la_bf16x4 v0 = *(const la_bf16x4*)vr, v1 = *(const la_bf16x4*)(vr + 16);
+                const la_bf16x8 vv = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+                acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, ph, acc[db], 0, 0, 0);
+                acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, pl, acc[db], 0, 0, 0);
+            }
+        __syncthreads();
+    }
+    l += __shfl_xor(l, 16, HB_WAVE);
+    l += __shfl_xor(l, 32, HB_WAVE);
+    if (!head) return;
+    // acc[db][i]: number 16 db + 4 g + i of head n's sum
+    const size_t row = (size_t)t * H + h;
+    if (splits == 1) {
+        float w = l > 0.f ? 1.0f / l : 0.f;
+        if (gate) w *= 1.0f / (1.0f + expf(-gate[(size_t)t * gate_ld + h]));
+#pragma unroll
+        for (int db = 0; db < RB; ++db)
+            if (db < rblocks) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) out[row * rank + db * 16 + 4 * g + i] = hb_from_float<bf16>(acc[db][i] * w);
+            }
+    } else {
+        float* pa = part_acc + (row * splits + split) * rank;
+#pragma unroll
+        for (int db = 0; db < RB; ++db)
+            if (db < rblocks) *(la_f32x4*)(pa + db * 16 + 4 * g) = acc[db];
+        if (g == 0) {
+            part_ml[(row * splits + split) * 2] = m;
+            part_ml[(row * splits + split) * 2 + 1] = l;
+        }
+    }
+}
+
+// out[row, :] = sum over the ranges (in order) of their sums, brought to one maximum, over the summed
+// denominators, times sigmoid(gate). One wave a (token, head).
+__global__ void __launch_bounds__(HB_WAVE)
+latent_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml, bf16* __restrict__ out,
+                    const float* __restrict__ gate, int gate_ld, int H, int rank, int splits) {
+    const size_t row = blockIdx.x;
+    const int lane = threadIdx.x;
+    float m = -INFINITY;
+    for (int s = 0; s < splits; ++s) m = fmaxf(m, part_ml[(row * splits + s) * 2]);
+    float l = 0.f;
+    for (int s = 0; s < splits; ++s) {
+        const float ms = part_ml[(row * splits + s) * 2];
+        if (ms > -INFINITY) l += part_ml[(row * splits + s) * 2 + 1] * expf(ms - m);
+    }
+    float w = l > 0.f ? 1.0f / l : 0.f;
+    if (gate) w *= 1.0f / (1.0f + expf(-gate[(row / H) * gate_ld + row % H]));
+    for (int d = lane; d < rank; d += HB_WAVE) {
+        float a = 0.f;
+        for (int s = 0; s < splits; ++s) {
+            const float ms = part_ml[(row * splits + s) * 2];
+            if (ms > -INFINITY) a = fmaf(part_acc[(row * splits + s) * rank + d], expf(ms - m), a);
+        }
+        out[row * rank + d] = hb_from_float<bf16>(a * w);
+    }
+}
+
+extern "C" int hb_latent_attention_mfma(const float* q_full, const void* pages, void* out, float* part_acc,
+                                        float* part_ml, const float* gate, int gate_ld, const int* positions,
+                                        const int* seq_of, const int* slots, const int* page_table, int max_pages,
+                                        int page_size, int T, int H, int rank, int rot, float scale, int splits,
+                                        int chunks_per_split, hipStream_t stream) {
+    HB_REQUIRE(T > 0 && H > 0, "latent attention: empty input");
+    HB_REQUIRE(rank > 0 && rank % 16 == 0 && rank <= 512 && (rank + rot) % 32 == 0 && rank + rot <= 640,
+               "latent attention: the matrix-core kernel takes a latent in steps of 16 up to 512 whose row is a multiple of 32, not %d + %d", rank, rot);
+    HB_REQUIRE(page_size % LA_CHUNK == 0, "latent attention: pages of %d positions", page_size);
+    HB_REQUIRE(splits >= 1 && splits <= 65535 && chunks_per_split >= 1, "latent attention: %d ranges", splits);
+    HB_REQUIRE(splits == 1 || (part_acc && part_ml), "latent attention: ranges need scratch");
+    const long long blocks = (long long)T * ((H + 15) / 16);
+    HB_REQUIRE(blocks < (1ll << 31), "latent attention: too many tokens for the grid");
+    const dim3 grid((unsigned)blocks, splits);
+#define LA_LAUNCH(RBV, KSV)                                                                                      \
+    latent_attention_mfma_kernel<RBV, KSV><<<grid, HB_WAVE, 0, stream>>>(                                          \
+        q_full, (const bf16*)pages, (bf16*)out, part_acc, part_ml, gate, gate_ld, positions, seq_of, slots,      \
+        page_table, max_pages, page_size, H, rank, rot, scale, splits, chunks_per_split)
+    if (rank <= 128 && rank + rot <= 256) LA_LAUNCH(8, 8);
+    else if (rank <= 256 && rank + rot <= 384) LA_LAUNCH(16, 12);
+    else LA_LAUNCH(32, 20);
+#undef LA_LAUNCH
+    HB_CHECK_LAUNCH("latent_attention_mfma");
+    if (splits > 1) {
+        latent_merge_kernel<<<(unsigned)((long long)T * H), HB_WAVE, 0, stream>>>(part_acc, part_ml, (bf16*)out, gate, gate_ld, H, rank, splits);
+        HB_CHECK_LAUNCH("latent_merge");
+    }
+    return 0;
+}

@@ -65,3 +65,47 @@ def latent_attention_plain(q_full, meta, cache, out, gate, gate_off, H, rank, ro
              dtype_code(cache.k), gate_ptr, gate_ld, meta.positions.data_ptr(), meta.seq_of.data_ptr(),
              meta.slots.data_ptr(), cache.page_table.data_ptr(), cache.page_table.shape[1], cache.page_size, T, H,
              rank, rot, float(scale), _stream())
+
+
+CHUNK = 32
+TARGET_WAVES = 1024        # a decode step's keys are cut into ranges until about this many waves run
+
+
+def mfma_takes(cache, rank, rot):
+    """True if the matrix-core kernel takes this latent: bfloat16 rows, rank in steps of 16 up to 512,
+    rows in steps of 32."""
+    return (cache.k.dtype == torch.bfloat16 and rank % 16 == 0 and 0 < rank <= 512 and (rank + rot) % 32 == 0
+            and cache.page_size % CHUNK == 0)
+
+
+def latent_attention_mfma(q_full, meta, cache, out, gate, gate_off, H, rank, rot, scale, buffer):
+    """latent_attention_plain on the matrix cores (see mfma_takes). A step of one token a sequence cuts its
+    keys into ranges, whose partial results lie in scratch from `buffer(name, shape, dtype)`."""
+    T = q_full.shape[0]
+    _check(q_full, "q_full", torch.float32, (T, H * (rank + rot)))
+    _check(out, "out", torch.bfloat16, (T, H * rank))
+    _check_pages(meta, cache, T, rank + rot)
+    if not mfma_takes(cache, rank, rot):
+        raise BackendError(f"latent attention: the matrix-core kernel does not take a latent of {rank} + {rot}")
+    gate_ptr, gate_ld = None, 0
+    if gate is not None:
+        _check(gate, "gate", torch.float32, (T, None))
+        gate_ld = gate.shape[1]
+        if gate_off < 0 or gate_off + H > gate_ld:
+            raise BackendError("latent attention: the gate's columns lie outside its rows")
+        gate_ptr = gate.data_ptr() + 4 * gate_off
+    splits, per = 1, 1 << 30
+    if meta.max_new == 1:
+        # the grid must not depend on the contexts themselves (a recorded step is replayed at others of its bucket)
+        chunks = -(-max(meta.context_bucket, meta.max_context) // CHUNK)
+        blocks = T * ((H + 15) // 16)
+        splits = max(1, min(TARGET_WAVES // blocks, -(-chunks // 4)))
+        per = -(-chunks // splits)
+    part_acc = part_ml = None
+    if splits > 1:
+        part_acc = buffer("latent_partial", (T * H * splits, rank), torch.float32)
+        part_ml = buffer("latent_partial_ml", (T * H * splits, 2), torch.float32)
+    lib.call("attention_latent", "hb_latent_attention_mfma", q_full.data_ptr(), cache.k.data_ptr(), out.data_ptr(),
+             _ptr(part_acc), _ptr(part_ml), gate_ptr, gate_ld, meta.positions.data_ptr(), meta.seq_of.data_ptr(),
+             meta.slots.data_ptr(), cache.page_table.data_ptr(), cache.page_table.shape[1], cache.page_size, T, H,
+             rank, rot, float(scale), splits, per, _stream())

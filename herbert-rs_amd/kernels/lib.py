@@ -40,6 +40,7 @@ SIGNATURES = {
     },
     "attention_latent": {
         "hb_latent_write": [_P, _I, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
+        "hb_latent_attention_mfma": [_P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
         "hb_latent_attention_plain": [_P, _P, _P, _I, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P],
     },
     "moe": {

@@ -95,8 +95,13 @@ class LatentAttention(Part):
             ops.gemm_plain_batched(proj, self.uk_t, q_full, T, self.rank, self.dim, self.width, self.dim,
                                    H * self.row, H, self.dim + self.rot_dim, self.rank * self.dim, self.row)
         mixed = rt.buffer("latent_mixed", (T, H * self.rank))
-        latent.latent_attention_plain(q_full, ctx.meta, kv, mixed, proj if self.gated else None,
-                                      self.q_width + self.row, H, self.rank, self.rot_dim, self.scale)
+        gate = proj if self.gated else None
+        if latent.mfma_takes(kv, self.rank, self.rot_dim):
+            latent.latent_attention_mfma(q_full, ctx.meta, kv, mixed, gate, self.q_width + self.row, H, self.rank,
+                                         self.rot_dim, self.scale, rt.buffer)
+        else:
+            latent.latent_attention_plain(q_full, ctx.meta, kv, mixed, gate, self.q_width + self.row, H, self.rank,
+                                          self.rot_dim, self.scale)
         # a head's summed latents through its W_uv
         attn = rt.buffer("latent_attn", (T, H * self.vdim))
         if cores:
