@@ -99,19 +99,36 @@ extern "C" int hb_conv_silu(const float* proj, int ld, const float* taps, float*
 //   S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q        (o sees the token's own write)
 // with g = exp(-exp(A_log[h]) * softplus(a + dt_bias[h])) and beta = sigmoid(b), a and b columns of
 // the projection's row. The columns of S never meet, and the tokens are a chain: the kernel is as
-// fast as one token's step is short. A column is held by LPC lanes (each 32 of its D numbers, in
-// registers; LPC = 1, 2, 4 or 8 for D up to 256), a wave holds 64 / LPC columns and walks the
-// sequence's tokens; the two dot products a token are summed over a column's lanes by LPC - 1
-// exchanges. The token ahead is loaded while the present one is worked on, and g and beta of a
-// token do not wait for the chain.
+// fast as one token's step is short. A column is held by LPC lanes (each 16 of its D numbers, in
+// registers; LPC = 1 .. 16 for D up to 256), a wave holds 64 / LPC columns and walks the sequence's
+// tokens; a workgroup is one wave, so that a head's columns spread over many CUs. The two dot
+// products a token are summed over a column's lanes by exchanges within a row of 16 lanes. What a
+// token needs (k, q, its values, g and beta, which do not wait for the chain) comes from a ring in
+// LDS that is filled 16 to 24 tokens ahead: a token's own loads would each cost the memory's latency.
 // qkv rows: [kv_heads x D queries | kv_heads x D keys | heads x V values]; head h reads the
 // query and key of kv head h / (heads / kv_heads).
-#define DELTA_PER 32
+#define DELTA_PER 16
+#define DELTA_SUB 8          // tokens that are loaded together
+#define DELTA_RING_OF(LPC) ((LPC) >= 16 ? 3 : 4)     // such groups in the ring (three where four would not fit 64 KB of LDS)
 
+__device__ __forceinline__ float delta_dpp(float v, const int ctrl) {
+    // (a lane reads another lane's value: ctrl names which, within rows of 16 lanes)
+    switch (ctrl) {
+        case 0: return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));    // lane ^ 1
+        case 1: return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));    // lane ^ 2
+        case 2: return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));   // 7 - lane of each 8
+        default: return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));  // 15 - lane of each 16
+    }
+}
+
+// the sum over the LPC lanes of a column, in every one of them (after each step all lanes of a
+// group of 2, 4, 8, 16 hold that group's sum, so a mirrored lane of the other half holds the other half's)
 template <int LPC>
 __device__ __forceinline__ float delta_column_sum(float v) {
-#pragma unroll
-    for (int off = 1; off < LPC; off <<= 1) v += __shfl_xor(v, off, HB_WAVE);
+    if (LPC >= 2) v += delta_dpp(v, 0);
+    if (LPC >= 4) v += delta_dpp(v, 1);
+    if (LPC >= 8) v += delta_dpp(v, 2);
+    if (LPC >= 16) v += delta_dpp(v, 3);
     return v;
 }
 
@@ -122,76 +139,133 @@ gated_delta_kernel(const float* __restrict__ qkv, int C, const float* __restrict
                    float* __restrict__ state, const int* __restrict__ seq_starts, const int* __restrict__ slots,
                    float* __restrict__ out, int kv_heads, int heads, int D, int V) {
     constexpr int COLS = HB_WAVE / LPC;
+    constexpr int DP = LPC * DELTA_PER;                 // D rounded up to what the lanes hold
+    constexpr int DELTA_RING = DELTA_RING_OF(LPC);
+    constexpr int SLOTS = DELTA_SUB * DELTA_RING;
+    constexpr int KQ4 = DELTA_SUB * DP / 2;             // float4 of k and q a group of tokens
+    constexpr int KQ_PER_LANE = (KQ4 + HB_WAVE - 1) / HB_WAVE;
+    constexpr int V_PER_LANE = (DELTA_SUB * COLS + HB_WAVE - 1) / HB_WAVE;
+    __shared__ __attribute__((aligned(16))) float kq_ring[SLOTS][2 * DP];
+    __shared__ float v_ring[SLOTS][COLS];
+    __shared__ float gb_ring[SLOTS][2];
     const int seq = blockIdx.x, h = blockIdx.y;
     const int lane = threadIdx.x;
-    const int part = lane % LPC;                       // which 32 of the column's D numbers
-    const int col = blockIdx.z * COLS + lane / LPC;
+    const int part = lane % LPC;                       // which 16 of the column's D numbers
+    const int lcol = lane / LPC;
+    const int col0 = blockIdx.z * COLS;
+    const int col = col0 + lcol;
     const bool live = col < V;
     const int d0 = part * DELTA_PER;
     const int kvh = h / (heads / kv_heads);
     const int first = seq_starts[seq], last = seq_starts[seq + 1];
+    const int n_groups = (last - first + DELTA_SUB - 1) / DELTA_SUB;
     float* S_mem = state + ((size_t)slots[seq] * heads + h) * D * V + col;
     float S[DELTA_PER];
-    // (numbers beyond D are zeros and stay zeros: their k and q are loaded as zeros)
+    // (numbers beyond D are zeros and stay zeros: their k and q are zeros in the ring)
 #pragma unroll
     for (int i = 0; i < DELTA_PER; ++i) S[i] = (live && d0 + i < D) ? S_mem[(size_t)(d0 + i) * V] : 0.f;
     const float rate = -expf(A_log[h]);
     const float bias = dt_bias[h];
-    const int q_at = kvh * D + d0, k_at = (kv_heads + kvh) * D + d0, v_at = 2 * kv_heads * D + h * V;
-    const bool whole = d0 + DELTA_PER <= D && (D % 4) == 0 && (C % 4) == 0;      // 16-byte loads of this lane's 32
+    const int q_at = kvh * D, k_at = (kv_heads + kvh) * D, v_at = 2 * kv_heads * D + h * V;
+    const bool vec = (D % 4) == 0 && (C % 4) == 0;
 
-    float kn[DELTA_PER], qn[DELTA_PER], vn = 0.f, an = 0.f, bn = 0.f;
-    auto load = [&](int t) {
-        const float* row = qkv + (size_t)t * C;
-        if (whole) {
+    float4 kq_regs[KQ_PER_LANE];
+    float v_regs[V_PER_LANE], g_reg = 0.f, beta_reg = 0.f;
+    // group p of the sequence's tokens from memory into registers ...
+    auto fetch = [&](int p) {
+        const int t0 = first + p * DELTA_SUB;
 #pragma unroll
-            for (int i = 0; i < DELTA_PER; i += 4) {
-                const float4 kk = *(const float4*)(row + k_at + i);
-                const float4 qq = *(const float4*)(row + q_at + i);
-                kn[i] = kk.x, kn[i + 1] = kk.y, kn[i + 2] = kk.z, kn[i + 3] = kk.w;
-                qn[i] = qq.x, qn[i + 1] = qq.y, qn[i + 2] = qq.z, qn[i + 3] = qq.w;
+        for (int j = 0; j < KQ_PER_LANE; ++j) {
+            const int idx = j * HB_WAVE + lane;
+            const int i = idx / (DP / 2), f = idx % (DP / 2);        // token of the group, float4 of its [k | q]
+            const int d = 4 * (f % (DP / 4));
+            float4 r = float4{0.f, 0.f, 0.f, 0.f};
+            if (idx < KQ4 && t0 + i < last) {
+                const float* src = qkv + (size_t)(t0 + i) * C + (f < DP / 4 ? k_at : q_at) + d;
+                if (vec && d + 3 < D) {
+                    r = *(const float4*)src;
+                } else {
+                    if (d < D) r.x = src[0];
+                    if (d + 1 < D) r.y = src[1];
+                    if (d + 2 < D) r.z = src[2];
+                    if (d + 3 < D) r.w = src[3];
+                }
             }
-        } else {
-#pragma unroll
-            for (int i = 0; i < DELTA_PER; ++i) {
-                kn[i] = d0 + i < D ? row[k_at + i] : 0.f;
-                qn[i] = d0 + i < D ? row[q_at + i] : 0.f;
-            }
+            kq_regs[j] = r;
         }
-        vn = live ? row[v_at + col] : 0.f;
-        an = proj[(size_t)t * ld + a_off + h];
-        bn = proj[(size_t)t * ld + b_off + h];
+#pragma unroll
+        for (int j = 0; j < V_PER_LANE; ++j) {
+            const int idx = j * HB_WAVE + lane;
+            const int i = idx / COLS, c = idx % COLS;
+            v_regs[j] = (idx < DELTA_SUB * COLS && t0 + i < last && col0 + c < V)
+                            ? qkv[(size_t)(t0 + i) * C + v_at + col0 + c] : 0.f;
+        }
+        if (lane < DELTA_SUB && t0 + lane < last) {
+            const float z = proj[(size_t)(t0 + lane) * ld + a_off + h] + bias;
+            const float softplus = z > 20.f ? z : log1pf(expf(z));
+            g_reg = expf(rate * softplus);
+            beta_reg = 1.0f / (1.0f + expf(-proj[(size_t)(t0 + lane) * ld + b_off + h]));
+        }
     };
-    if (first < last) load(first);
-    for (int t = first; t < last; ++t) {
-        float kc[DELTA_PER], qc[DELTA_PER];
+    // ... and from the registers into the ring
+    auto stash = [&](int p) {
+        const int s0 = (p % DELTA_RING) * DELTA_SUB;
 #pragma unroll
-        for (int i = 0; i < DELTA_PER; ++i) {
-            kc[i] = kn[i];
-            qc[i] = qn[i];
+        for (int j = 0; j < KQ_PER_LANE; ++j) {
+            const int idx = j * HB_WAVE + lane;
+            if (idx < KQ4) *(float4*)&kq_ring[s0 + idx / (DP / 2)][4 * (idx % (DP / 2))] = kq_regs[j];
         }
-        const float vc = vn;
-        const float z = an + bias;
-        const float softplus = z > 20.f ? z : log1pf(expf(z));
-        const float g = expf(rate * softplus);
-        const float beta = 1.0f / (1.0f + expf(-bn));
-        if (t + 1 < last) load(t + 1);
-        float dot = 0.f;
 #pragma unroll
-        for (int i = 0; i < DELTA_PER; ++i) {
-            S[i] *= g;
-            dot = fmaf(S[i], kc[i], dot);
+        for (int j = 0; j < V_PER_LANE; ++j) {
+            const int idx = j * HB_WAVE + lane;
+            if (idx < DELTA_SUB * COLS) v_ring[s0 + idx / COLS][idx % COLS] = v_regs[j];
         }
-        dot = delta_column_sum<LPC>(dot);
-        const float u = beta * (vc - dot);
-        float o = 0.f;
+        if (lane < DELTA_SUB) {
+            gb_ring[s0 + lane][0] = g_reg;
+            gb_ring[s0 + lane][1] = beta_reg;
+        }
+    };
+    for (int p = 0; p < DELTA_RING - 1 && p < n_groups; ++p) {
+        fetch(p);
+        stash(p);
+    }
+    __syncthreads();
+    for (int p = 0; p < n_groups; ++p) {
+        const bool ahead = p + DELTA_RING - 1 < n_groups;
+        if (ahead) fetch(p + DELTA_RING - 1);
+        const int s0 = (p % DELTA_RING) * DELTA_SUB;
+        const int t0 = first + p * DELTA_SUB;
+        const int n = last - t0 < DELTA_SUB ? last - t0 : DELTA_SUB;
+        for (int i = 0; i < n; ++i) {
+            float kc[DELTA_PER], qc[DELTA_PER];
 #pragma unroll
-        for (int i = 0; i < DELTA_PER; ++i) {
-            S[i] = fmaf(kc[i], u, S[i]);
-            o = fmaf(S[i], qc[i], o);
+            for (int e = 0; e < DELTA_PER; e += 4) {
+                const float4 kk = *(const float4*)&kq_ring[s0 + i][d0 + e];
+                const float4 qq = *(const float4*)&kq_ring[s0 + i][DP + d0 + e];
+                kc[e] = kk.x, kc[e + 1] = kk.y, kc[e + 2] = kk.z, kc[e + 3] = kk.w;
+                qc[e] = qq.x, qc[e + 1] = qq.y, qc[e + 2] = qq.z, qc[e + 3] = qq.w;
+            }
+            const float vc = v_ring[s0 + i][lcol];
+            const float g = gb_ring[s0 + i][0], beta = gb_ring[s0 + i][1];
+            float dot = 0.f;
+#pragma unroll
+            for (int e = 0; e < DELTA_PER; ++e) {
+                S[e] *= g;
+                dot = fmaf(S[e], kc[e], dot);
+            }
+            dot = delta_column_sum<LPC>(dot);
+            const float u = beta * (vc - dot);
+            float o = 0.f;
+#pragma unroll
+            for (int e = 0; e < DELTA_PER; ++e) {
+                S[e] = fmaf(kc[e], u, S[e]);
+                o = fmaf(S[e], qc[e], o);
+            }
+            o = delta_column_sum<LPC>(o);
+            if (live && part == 0) out[(size_t)(t0 + i) * heads * V + h * V + col] = o;
         }
-        o = delta_column_sum<LPC>(o);
-        if (live && part == 0) out[(size_t)t * heads * V + h * V + col] = o;
+        if (ahead) stash(p + DELTA_RING - 1);           // (the place of the group before this one)
+        __syncthreads();
     }
     if (live) {
 #pragma unroll
@@ -208,7 +282,7 @@ extern "C" int hb_gated_delta(const float* qkv, int C, const float* proj, int ld
     HB_REQUIRE(D > 0 && D <= 256, "delta rule: keys of %d, the kernel takes 1 to 256", D);
     HB_REQUIRE(V > 0 && C == 2 * kv_heads * D + heads * V, "delta rule: %d channels do not fit the heads", C);
     HB_REQUIRE(B <= 65535 && heads <= 65535, "delta rule: too many sequences or heads for the grid");
-    const int lpc = D <= 32 ? 1 : D <= 64 ? 2 : D <= 128 ? 4 : 8;
+    const int lpc = D <= 16 ? 1 : D <= 32 ? 2 : D <= 64 ? 4 : D <= 128 ? 8 : 16;
     const int cols = HB_WAVE / lpc;
     const dim3 grid(B, heads, (V + cols - 1) / cols);
 #define HB_DELTA(L)                                                                                               \
@@ -217,7 +291,8 @@ extern "C" int hb_gated_delta(const float* qkv, int C, const float* proj, int ld
     if (lpc == 1) HB_DELTA(1);
     else if (lpc == 2) HB_DELTA(2);
     else if (lpc == 4) HB_DELTA(4);
-    else HB_DELTA(8);
+    else if (lpc == 8) HB_DELTA(8);
+    else HB_DELTA(16);
 #undef HB_DELTA
     HB_CHECK_LAUNCH("gated_delta");
     return 0;
