@@ -208,7 +208,8 @@ extern "C" int hb_latent_attention_plain(const float* q_full, const void* pages,
 // and low, so that it keeps 16 bits of mantissa. The sums are float32, and so are the softmax and its
 // state, which are a lane's own (a lane holds scores of one head only). Weighted sums: O^T = V^T P^T
 // with the weights again as high and low halves (they are never rounded to 8 bits), and V^T, the
-// chunk's first `rank` numbers a key with the keys along a row, transposed through LDS. The 32 keys
+// chunk's first `rank` numbers a key with the keys along a row, written to LDS from the registers
+// that hold them as the scores' operands. The 32 keys
 // of a product stand in the order in which the scores' lanes hold them (4 g + i of the first block of
 // 16, then of the second), so the weights go from the scores' registers into the next product as they
 // are. With more than one range a token the unnormalised sums, maxima and denominators go to scratch
@@ -281,6 +282,11 @@ latent_attention_mfma_kernel(const float* __restrict__ q_full, const bf16* __res
                     const la_bf16x8 kv = *(const la_bf16x8*)(krow + 32 * ks);
                     s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kv, qh[ks], s[kb], 0, 0, 0);
                     s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kv, ql[ks], s[kb], 0, 0, 0);
+                    // the same numbers are the key's part of V^T: key 16 kb + n, numbers 32 ks + 8 g + e
+                    if (32 * ks + 8 * g < rank) {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) Vt[(32 * ks + 8 * g + e) * LA_VT_STRIDE + 16 * kb + n] = kv[e];
+                    }
                 }
         }
         // s[kb][i]: key j0 + 16 kb + 4 g + i against head n
@@ -315,16 +321,6 @@ latent_attention_mfma_kernel(const float* __restrict__ q_full, const bf16* __res
         for (int db = 0; db < RB; ++db)
 #pragma unroll
             for (int i = 0; i < 4; ++i) acc[db][i] *= corr;
-        // V^T into LDS: lane: key lane % 32, 8 numbers of it at a time
-        {
-            const int kk = lane & 31;
-            const bf16* vrow = chunk + (size_t)kk * kd;
-            for (int c8 = lane >> 5; c8 < rank / 8; c8 += 2) {
-                const la_bf16x8 v = *(const la_bf16x8*)(vrow + 8 * c8);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) Vt[(8 * c8 + e) * LA_VT_STRIDE + kk] = v[e];
-            }
-        }
         __syncthreads();
 #pragma unroll
         for (int db = 0; db < RB; ++db)
@@ -370,21 +366,18 @@ latent_merge_kernel(const float* __restrict__ part_acc, const float* __restrict_
                     const float* __restrict__ gate, int gate_ld, int H, int rank, int splits) {
     const size_t row = blockIdx.x;
     const int lane = threadIdx.x;
-    float m = -INFINITY;
-    for (int s = 0; s < splits; ++s) m = fmaxf(m, part_ml[(row * splits + s) * 2]);
-    float l = 0.f;
-    for (int s = 0; s < splits; ++s) {
-        const float ms = part_ml[(row * splits + s) * 2];
-        if (ms > -INFINITY) l += part_ml[(row * splits + s) * 2 + 1] * expf(ms - m);
-    }
+    // lane s holds range s's share (at most 64 ranges)
+    const bool has = lane < splits;
+    const float ms = has ? part_ml[(row * splits + lane) * 2] : -INFINITY;
+    const float ls = has ? part_ml[(row * splits + lane) * 2 + 1] : 0.f;
+    const float m = hb_wave_max(ms);
+    const float ws = ms > -INFINITY ? expf(ms - m) : 0.f;
+    const float l = hb_wave_sum(ls * ws);
     float w = l > 0.f ? 1.0f / l : 0.f;
     if (gate) w *= 1.0f / (1.0f + expf(-gate[(row / H) * gate_ld + row % H]));
     for (int d = lane; d < rank; d += HB_WAVE) {
         float a = 0.f;
-        for (int s = 0; s < splits; ++s) {
-            const float ms = part_ml[(row * splits + s) * 2];
-            if (ms > -INFINITY) a = fmaf(part_acc[(row * splits + s) * rank + d], expf(ms - m), a);
-        }
+        for (int s = 0; s < splits; ++s) a = fmaf(part_acc[(row * splits + s) * rank + d], __shfl(ws, s, HB_WAVE), a);
         out[row * rank + d] = hb_from_float<bf16>(a * w);
     }
 }
@@ -398,7 +391,7 @@ extern "C" int hb_latent_attention_mfma(const float* q_full, const void* pages, 
     HB_REQUIRE(rank > 0 && rank % 16 == 0 && rank <= 512 && (rank + rot) % 32 == 0 && rank + rot <= 640,
                "latent attention: the matrix-core kernel takes a latent in steps of 16 up to 512 whose row is a multiple of 32, not %d + %d", rank, rot);
     HB_REQUIRE(page_size % LA_CHUNK == 0, "latent attention: pages of %d positions", page_size);
-    HB_REQUIRE(splits >= 1 && splits <= 65535 && chunks_per_split >= 1, "latent attention: %d ranges", splits);
+    HB_REQUIRE(splits >= 1 && splits <= HB_WAVE && chunks_per_split >= 1, "latent attention: %d ranges, the kernels take 1 to 64", splits);
     HB_REQUIRE(splits == 1 || (part_acc && part_ml), "latent attention: ranges need scratch");
     const long long blocks = (long long)T * ((H + 15) / 16);
     HB_REQUIRE(blocks < (1ll << 31), "latent attention: too many tokens for the grid");

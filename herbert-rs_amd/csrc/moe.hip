@@ -267,11 +267,23 @@ extern "C" int hb_moe_activate(const float* gu, void* act, int act_dtype, int ro
 __global__ void moe_combine_kernel(const float* __restrict__ y, const float* __restrict__ weight,
                                    const int* __restrict__ row_of, float* __restrict__ x, int top, int H) {
     const int t = blockIdx.x;
-    for (int i = threadIdx.x; i < H; i += blockDim.x) {
-        float s = 0.f;
-        for (int j = 0; j < top; ++j)
-            s = fmaf(weight[(size_t)t * top + j], y[(size_t)row_of[(size_t)t * top + j] * H + i], s);
-        x[(size_t)t * H + i] += s;
+    // (a token's rows and weights once, eight at a time, then whole rows)
+    for (int j0 = 0; j0 < top; j0 += 8) {
+        const float* rows[8];
+        float w[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const bool in = j0 + j < top;
+            rows[j] = y + (size_t)row_of[(size_t)t * top + (in ? j0 + j : 0)] * H;
+            w[j] = in ? weight[(size_t)t * top + j0 + j] : 0.f;
+        }
+        for (int i = threadIdx.x; i < H; i += blockDim.x) {
+            float s = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                if (j0 + j < top) s = fmaf(w[j], rows[j][i], s);
+            x[(size_t)t * H + i] += s;
+        }
     }
 }
 
@@ -289,10 +301,12 @@ extern "C" int hb_moe_combine(const float* y, const float* weight, const int* ro
 // g * a_group_off on) with its own matrix W[g] [N, K] into columns of C from g * c_group_off on.
 // The rows of a group come as a list of tiles (group, first row, rows <= 64) or, without a list, as
 // every group's ceil(M / 64) tiles of the same M rows (heads that each have a matrix of their own).
-// A workgroup is four waves on one tile of 64 rows; a wave holds two blocks of 16 weight rows
+// A workgroup is four waves on one tile of 64 rows; a wave holds four blocks of 16 weight rows
 // against up to four blocks of 16 activation rows (the blocks beyond the tile's rows are skipped, so
-// a tile of a few rows costs little more than streaming its weights). Operands go from memory
-// straight into the lanes: lane l of an operand holds 8 consecutive k of row l % 16 from k0 + 8 (l / 16).
+// a tile of a few rows costs little more than streaming its weights). The weights go from memory
+// straight into the lanes (lane l of an operand holds 8 consecutive k of row l % 16 from k0 + 8 (l / 16)),
+// a stage ahead of their products; the tile's activations, which the four waves share, through two
+// stages in LDS.
 // An output is summed over k in the same order whatever else the tile holds.
 // EPI 0: float32 C. EPI 1: bfloat16 C. EPI 2: W[g] is [2 F, K], gate rows then up rows; a wave's two
 // blocks are 16 gate rows and the 16 up rows that go with them, and C [*, F] bfloat16 receives
@@ -300,9 +314,140 @@ extern "C" int hb_moe_combine(const float* y, const float* weight, const int* ro
 typedef __bf16 hb_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float hb_f32x4 __attribute__((ext_vector_type(4)));
 
+#define GM_KSTEP 64           // k a stage of the activations' ring in LDS
+
 template <int EPI>
 __global__ void __launch_bounds__(256)
 grouped_mfma_kernel(const bf16* __restrict__ A, int lda, size_t a_group_off, const bf16* __restrict__ W, int N,
+                    int K, void* __restrict__ Cv, int ldc, size_t c_group_off, const int* __restrict__ order,
+                    int top, const int* __restrict__ tile_group, const int* __restrict__ tile_row0,
+                    const int* __restrict__ tile_rows, int M, int m_tiles, float limit, float alpha) {
+    // the tile's activations, a stage of 64 k at a time, as 16-byte pieces [k piece][row]: a wave's operand
+    // (16 rows of one piece) is 256 contiguous bytes
+    __shared__ __attribute__((aligned(16))) hb_bf16x8 a_lds[2][GM_KSTEP / 8][MOE_TILE_M];
+    int group, row0, rows;
+    if (tile_group) {
+        group = tile_group[blockIdx.y];
+        if (group < 0) return;
+        row0 = tile_row0[blockIdx.y];
+        rows = tile_rows[blockIdx.y];
+    } else {
+        group = blockIdx.y / m_tiles;
+        row0 = (blockIdx.y % m_tiles) * MOE_TILE_M;
+        rows = M - row0 < MOE_TILE_M ? M - row0 : MOE_TILE_M;
+    }
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int r16 = lane & 15, g4 = lane >> 4;
+    const int F = N / 2;
+    const int out_cols = EPI == 2 ? F : N;
+    // the wave's output columns: 64 of them, or with EPI 2 32 (from 32 gate rows and the 32 up rows that go with them)
+    const int n0 = EPI == 2 ? (blockIdx.x * 4 + wave) * 32 : (blockIdx.x * 4 + wave) * 64;
+    const bool idle = n0 >= out_cols;            // (such a wave still helps to load the activations)
+    const bf16* Wg = W + (size_t)group * N * K;
+    const bf16* wrow[4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+        int n = (EPI == 2 ? (a < 2 ? n0 + 16 * a : F + n0 + 16 * (a - 2)) : n0 + 16 * a) + r16;
+        if (n >= N || idle) n = N - 1;               // (read a row that exists; its sums are not stored)
+        wrow[a] = Wg + (size_t)n * K + g4 * 8;
+    }
+    const int blocks = (rows + 15) / 16;
+    // what this thread brings of a stage: rows tid / 8 and 32 + tid / 8, piece tid % 8
+    const bf16* asrc[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        int m = 32 * j + tid / 8;
+        if (m >= rows) m = rows - 1;
+        const int src = top > 0 ? order[row0 + m] / top : row0 + m;
+        asrc[j] = A + (size_t)src * lda + (size_t)group * a_group_off + (tid % 8) * 8;
+    }
+    hb_f32x4 acc[4][4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) acc[a][b] = hb_f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int stages = (K + GM_KSTEP - 1) / GM_KSTEP;
+    hb_bf16x8 areg[2], wnext[2][4];
+    auto fetch = [&](int st) {
+        const int k0 = st * GM_KSTEP;
+        const bool tail = k0 + (tid % 8) * 8 >= K;          // (K in steps of 32: the last stage may be half)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) areg[j] = tail ? hb_bf16x8{} : *(const hb_bf16x8*)(asrc[j] + k0);
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+                wnext[h][a] = k0 + 32 * h < K ? *(const hb_bf16x8*)(wrow[a] + k0 + 32 * h) : hb_bf16x8{};
+    };
+    fetch(0);
+    for (int st = 0; st < stages; ++st) {
+        const int buf = st & 1;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) a_lds[buf][tid % 8][32 * j + tid / 8] = areg[j];
+        hb_bf16x8 wv[2][4];
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int a = 0; a < 4; ++a) wv[h][a] = wnext[h][a];
+        __syncthreads();          // the stage is in LDS (and the stage before the last has been read by all)
+        if (st + 1 < stages) fetch(st + 1);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            hb_bf16x8 xv[4];
+#pragma unroll
+            for (int b = 0; b < 4; ++b)
+                if (b < blocks) xv[b] = a_lds[buf][4 * h + g4][16 * b + r16];
+#pragma unroll
+            for (int b = 0; b < 4; ++b)
+                if (b < blocks) {
+#pragma unroll
+                    for (int a = 0; a < 4; ++a)
+                        acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[h][a], xv[b], acc[a][b], 0, 0, 0);
+                }
+        }
+    }
+    if (idle) return;
+    // lane: activation row b * 16 + r16, weight rows g4 * 4 + i of each block
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        const int m = b * 16 + r16;
+        if (b >= blocks || m >= rows) continue;
+        const size_t base = (size_t)(row0 + m) * ldc + (size_t)group * c_group_off;
+        if (EPI == 2) {
+            bf16* C = (bf16*)Cv;
+#pragma unroll
+            for (int a = 0; a < 2; ++a)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int n = n0 + 16 * a + g4 * 4 + i;
+                    if (n >= F) continue;
+                    const float g = fminf(acc[a][b][i], limit);
+                    const float u = fminf(fmaxf(acc[a + 2][b][i], -limit), limit);
+                    C[base + n] = hb_from_float<bf16>(g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+                }
+        } else {
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int n = n0 + 16 * a + g4 * 4 + i;
+                    if (n >= N) continue;
+                    if (EPI == 0)
+                        ((float*)Cv)[base + n] = acc[a][b][i];
+                    else
+                        ((bf16*)Cv)[base + n] = hb_from_float<bf16>(acc[a][b][i]);
+                }
+        }
+    }
+}
+
+// The same for tiles of few rows (decoding): no stage in LDS and no barrier, a wave holds two blocks
+// of weight rows, so that more waves stream the weights; every operand straight from memory.
+template <int EPI>
+__global__ void __launch_bounds__(256)
+grouped_mfma_stream_kernel(const bf16* __restrict__ A, int lda, size_t a_group_off, const bf16* __restrict__ W, int N,
                     int K, void* __restrict__ Cv, int ldc, size_t c_group_off, const int* __restrict__ order,
                     int top, const int* __restrict__ tile_group, const int* __restrict__ tile_row0,
                     const int* __restrict__ tile_rows, int M, int m_tiles, float limit, float alpha) {
@@ -401,7 +546,7 @@ grouped_mfma_kernel(const bf16* __restrict__ A, int lda, size_t a_group_off, con
 extern "C" int hb_grouped_mfma(const void* A, int lda, size_t a_group_off, const void* W, int N, int K, void* C,
                                int ldc, size_t c_group_off, int epi, const int* order, int top,
                                const int* tile_group, const int* tile_row0, const int* tile_rows, int n_tiles, int M,
-                               int groups, float limit, float alpha, hipStream_t stream) {
+                               int groups, float limit, float alpha, int few_rows, hipStream_t stream) {
     HB_REQUIRE(N > 0 && K > 0 && K % 32 == 0, "grouped product: K = %d must be a positive multiple of 32", K);
     HB_REQUIRE(lda % 8 == 0 && a_group_off % 8 == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0,
                "grouped product: operands must lie at multiples of 16 bytes");
@@ -414,8 +559,21 @@ extern "C" int hb_grouped_mfma(const void* A, int lda, size_t a_group_off, const
     }
     HB_REQUIRE(tiles > 0 && tiles <= 65535, "grouped product: %d row tiles exceed the grid", tiles);
     const int out_cols = epi == 2 ? N / 2 : N;
-    const int per_group = epi == 2 ? 64 : 128;
+    // few_rows: the tiles hold few rows each (the host knows how many rows there are to how many groups)
+    const int per_group = few_rows ? (epi == 2 ? 64 : 128) : (epi == 2 ? 128 : 256);
     const dim3 grid((out_cols + per_group - 1) / per_group, tiles);
+#define HB_GROUPED_STREAM(E)                                                                                        \
+    grouped_mfma_stream_kernel<E><<<grid, 256, 0, stream>>>((const bf16*)A, lda, a_group_off, (const bf16*)W, N, K, \
+                                                            C, ldc, c_group_off, order, top, tile_group, tile_row0,  \
+                                                            tile_rows, M, m_tiles, limit, alpha)
+    if (few_rows) {
+        if (epi == 0) HB_GROUPED_STREAM(0);
+        else if (epi == 1) HB_GROUPED_STREAM(1);
+        else HB_GROUPED_STREAM(2);
+        HB_CHECK_LAUNCH("grouped_mfma_stream");
+        return 0;
+    }
+#undef HB_GROUPED_STREAM
 #define HB_GROUPED(E)                                                                                               \
     grouped_mfma_kernel<E><<<grid, 256, 0, stream>>>((const bf16*)A, lda, a_group_off, (const bf16*)W, N, K, C, ldc, \
                                                      c_group_off, order, top, tile_group, tile_row0, tile_rows, M,   \

@@ -48,7 +48,7 @@ SIGNATURES = {
         "hb_moe_gemm_plain": [_P, _I, _P, _I, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _P],
         "hb_moe_activate": [_P, _P, _I, _I, _I, _F, _F, _P],
         "hb_moe_combine": [_P, _P, _P, _P, _I, _I, _I, _P],
-        "hb_grouped_mfma": [_P, _I, _SZ, _P, _I, _I, _P, _I, _SZ, _I, _P, _I, _P, _P, _P, _I, _I, _I, _F, _F, _P],
+        "hb_grouped_mfma": [_P, _I, _SZ, _P, _I, _I, _P, _I, _SZ, _I, _P, _I, _P, _P, _P, _I, _I, _I, _F, _F, _I, _P],
     },
     "attention_plain": {
         "hb_attention_plain": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],

@@ -90,6 +90,7 @@ def combine(y, routing, x):
 
 
 EPI_F32, EPI_BF16, EPI_GLU = 0, 1, 2
+FEW_ROWS = 16      # up to so many rows a group the kernel without a stage in LDS runs (decoding)
 
 
 def mfma_takes(K, lda, a_group_off=0):
@@ -118,11 +119,13 @@ def grouped_mfma(a, lda, a_group_off, w, c, ldc, c_group_off, epi, routing=None,
             raise BackendError("grouped product: one matrix an expert")
         lists = (r.order.data_ptr(), r.top if gather else 0, r.tile_expert.data_ptr(), r.tile_row0.data_ptr(),
                  r.tile_rows.data_ptr(), r.tiles, 0, 0)
+        few = r.T * r.top <= FEW_ROWS * G          # (on average; the kernels take any tile either way)
     else:
         rows_a = rows_c = M
         lists = (None, 0, None, None, None, 0, M, G)
+        few = M <= FEW_ROWS
     if (rows_a - 1) * lda + (G - 1) * a_group_off + K > a.numel() or \
             (rows_c - 1) * ldc + (G - 1) * c_group_off + out_cols > c.numel():
         raise BackendError("grouped product: an operand does not hold every row that is addressed")
     lib.call("moe", "hb_grouped_mfma", a.data_ptr(), lda, a_group_off, w.data_ptr(), N, K, c.data_ptr(), ldc,
-             c_group_off, epi, *lists, float(limit), float(alpha), _stream())
+             c_group_off, epi, *lists, float(limit), float(alpha), 1 if few else 0, _stream())
