@@ -67,46 +67,39 @@ moe_route_kernel(const float* __restrict__ logits, const float* __restrict__ bia
 }
 
 // ------------------------------------------------------------------------ group
-__global__ void moe_count_kernel(const int* __restrict__ chosen, int* __restrict__ counts, int A) {
-    __shared__ int red[16];
-    const int e = blockIdx.x;
-    int n = 0;
-    for (int a = threadIdx.x; a < A; a += blockDim.x) n += chosen[a] == e;
-    for (int off = HB_WAVE / 2; off > 0; off >>= 1) n += __shfl_xor(n, off, HB_WAVE);
-    if ((threadIdx.x & (HB_WAVE - 1)) == 0) red[threadIdx.x / HB_WAVE] = n;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        int total = 0;
-        for (int w = 0; w < (int)(blockDim.x / HB_WAVE); ++w) total += red[w];
-        counts[e] = total;
-    }
-}
-
 // Block e < E: the pairs of expert e, in the order of the pairs, to rows [first, first + count) and
 // the expert's tiles into the list; block E: the list's unused end. order[row] = pair,
-// row_of[pair] = row.
+// row_of[pair] = row. Every block counts all experts' pairs for itself (a histogram in LDS), so that
+// no kernel has to run before it.
 __global__ void __launch_bounds__(256)
-moe_place_kernel(const int* __restrict__ chosen, const int* __restrict__ counts, int* __restrict__ order,
+moe_place_kernel(const int* __restrict__ chosen, int* __restrict__ counts, int* __restrict__ order,
                  int* __restrict__ row_of, int* __restrict__ tile_expert, int* __restrict__ tile_row0,
                  int* __restrict__ tile_rows, int A, int E, int max_tiles) {
+    __shared__ int hist[HB_WAVE * MOE_MAX_E_PER_LANE];
     __shared__ int wave_n[4];
     __shared__ int base;
     const int e = blockIdx.x;
+    for (int i = threadIdx.x; i < E; i += blockDim.x) hist[i] = 0;
+    __syncthreads();
+    for (int a = threadIdx.x; a < A; a += blockDim.x) atomicAdd(&hist[chosen[a]], 1);
+    __syncthreads();
     int first = 0, tile0 = 0;
     for (int i = 0; i < (e < E ? e : E); ++i) {
-        first += counts[i];
-        tile0 += (counts[i] + MOE_TILE_M - 1) / MOE_TILE_M;
+        first += hist[i];
+        tile0 += (hist[i] + MOE_TILE_M - 1) / MOE_TILE_M;
     }
     if (e == E) {
         for (int i = tile0 + threadIdx.x; i < max_tiles; i += blockDim.x) tile_expert[i] = -1;
         return;
     }
-    const int count = counts[e];
+    const int count = hist[e];
+    if (threadIdx.x == 0) counts[e] = count;
     for (int i = threadIdx.x; i * MOE_TILE_M < count; i += blockDim.x) {
         tile_expert[tile0 + i] = e;
         tile_row0[tile0 + i] = first + i * MOE_TILE_M;
         tile_rows[tile0 + i] = count - i * MOE_TILE_M < MOE_TILE_M ? count - i * MOE_TILE_M : MOE_TILE_M;
     }
+    if (count == 0) return;
     if (threadIdx.x == 0) base = first;
     __syncthreads();
     const int lane = threadIdx.x & (HB_WAVE - 1), wave = threadIdx.x / HB_WAVE;
@@ -139,8 +132,6 @@ extern "C" int hb_moe_route(const float* logits, const float* bias, int* chosen,
     HB_REQUIRE(max_tiles >= (A + MOE_TILE_M - 1) / MOE_TILE_M + E, "moe: the tile list is too short");
     moe_route_kernel<<<T, HB_WAVE, 0, stream>>>(logits, bias, chosen, weight, E, top);
     HB_CHECK_LAUNCH("moe_route");
-    moe_count_kernel<<<E, 256, 0, stream>>>(chosen, counts, (int)A);
-    HB_CHECK_LAUNCH("moe_count");
     moe_place_kernel<<<E + 1, 256, 0, stream>>>(chosen, counts, order, row_of, tile_expert, tile_row0, tile_rows, (int)A, E, max_tiles);
     HB_CHECK_LAUNCH("moe_place");
     return 0;

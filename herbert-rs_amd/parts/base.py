@@ -152,6 +152,12 @@ class StepContext:
     next_block: Any = None           # set by the model: the block of the schedule's next entry, or None
     # (x, delta, mult): a sum that a block has left for the next block's norm to add to x (x += mult * delta)
     pending_sum: Any = None
+    # rows that hold nothing yet: a part whose last product is to add to exactly these rows stores there instead
+    fresh_rows: Any = None
+
+    def adds_to(self, x):
+        """False if x are the context's fresh rows (the part's product stores), True if it has to add."""
+        return not (self.fresh_rows is not None and self.fresh_rows.data_ptr() == x.data_ptr())
 
     def leave_norm(self, linear, x):
         """For a part, just before `linear` adds its last product into x: a NormedRows that product

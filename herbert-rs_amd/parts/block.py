@@ -102,9 +102,15 @@ class ParallelBlock(Part):
         # the two parts' outputs meet in rows of their own (free again: the norm above has taken the sum
         # of the layer before)
         total = ctx.rt.buffer("parallel_sum", tuple(x.shape), torch.float32)
-        ops.fill_u32(total, 0)
         ctx.handed = ctx.norm_ahead = None
+        # a mixer that can store its rows instead of adding them says so (`stores_fresh_rows`) and finds the
+        # rows in ctx.fresh_rows; for any other the rows are cleared first
+        if getattr(self.mixer, "stores_fresh_rows", False):
+            ctx.fresh_rows = total
+        else:
+            ops.fill_u32(total, 0)
         self.mixer.forward(ctx, h, total)
+        ctx.fresh_rows = None
         if self.feed_forward is not None:
             self.feed_forward.forward(ctx, h, total)
         nxt = ctx.next_block

@@ -37,6 +37,7 @@ def _rate_init(shape, gen, device, std, norm_std):
 @register("mixer", "gated_delta")
 class GatedDelta(Part):
     graph_safe = True
+    stores_fresh_rows = True     # its output projection stores into rows that hold nothing yet (StepContext.adds_to)
 
     def __init__(self, hidden_size, heads, kv_heads, dim, vdim, conv, eps, names, unit_eps=UNIT_EPS, shared=None):
         """names: q, k, v, q_conv, k_conv, v_conv, b, a, A_log, dt_bias, g, norm, o -> tensor names.
@@ -107,5 +108,6 @@ class GatedDelta(Part):
                               self.kv_heads, self.heads, self.dim, self.vdim)
         gated = rt.buffer("delta_gated", (T, self.heads * self.vdim))
         recurrent.gated_head_norm(o, proj, self.g_off, self.norm_w, gated, self.heads, self.vdim, self.eps)
-        left = ctx.leave_norm(self.o, x)
-        self.o.forward(gated, x, accumulate=True, leave=None if left is None else left.leave())
+        adds = ctx.adds_to(x)
+        left = ctx.leave_norm(self.o, x) if adds else None
+        self.o.forward(gated, x, accumulate=adds, leave=None if left is None else left.leave())

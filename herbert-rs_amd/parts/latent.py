@@ -25,6 +25,7 @@ from .registry import register
 @register("mixer", "latent_attention")
 class LatentAttention(Part):
     graph_safe = True
+    stores_fresh_rows = True     # its output projection stores into rows that hold nothing yet (StepContext.adds_to)
 
     def __init__(self, hidden_size, heads, dim, rot_dim, vdim, kv_rank, scale, eps, position, names, shared=None):
         """names: q, dkv, dkv_norm, uk, uv, g (None: no output gate), o -> tensor names. position: the
@@ -109,5 +110,6 @@ class LatentAttention(Part):
         else:
             ops.gemm_plain_batched(mixed, self.uv, attn, T, self.vdim, self.rank, H * self.rank, self.rank,
                                    H * self.vdim, H, self.rank, self.vdim * self.rank, self.vdim)
-        left = ctx.leave_norm(self.o, x)
-        self.o.forward(attn, x, accumulate=True, leave=None if left is None else left.leave())
+        adds = ctx.adds_to(x)
+        left = ctx.leave_norm(self.o, x) if adds else None
+        self.o.forward(attn, x, accumulate=adds, leave=None if left is None else left.leave())
