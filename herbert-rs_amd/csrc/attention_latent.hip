@@ -205,8 +205,9 @@ extern "C" int hb_latent_attention_plain(const float* q_full, const void* pages,
 // A wave takes 16 heads of one token (the rows of its matrix products) and a range of the keys, in
 // chunks of 32. Scores: S^T = K Q^T, the chunk's rows straight from memory as operands (a lane: one
 // key's 8 consecutive numbers), the query (times the scale) in registers as two bfloat16 halves, high
-// and low, so that it keeps 16 bits of mantissa. The sums are float32, and so are the softmax and its
-// state, which are a lane's own (a lane holds scores of one head only). Weighted sums: O^T = V^T P^T
+// and low, so that it keeps 16 bits of mantissa (with the high half alone a test with large queries
+// lost a digit). The sums are float32, and so are the softmax and its state, which are a lane's own
+// (a lane holds scores of one head only). Weighted sums: O^T = V^T P^T
 // with the weights again as high and low halves (they are never rounded to 8 bits), and V^T, the
 // chunk's first `rank` numbers a key with the keys along a row, written to LDS from the registers
 // that hold them as the scores' operands. The 32 keys
@@ -214,7 +215,7 @@ extern "C" int hb_latent_attention_plain(const float* q_full, const void* pages,
 // 16, then of the second), so the weights go from the scores' registers into the next product as they
 // are. With more than one range a token the unnormalised sums, maxima and denominators go to scratch
 // and a second kernel joins them in the ranges' order.
-// Sizes: rank a multiple of 16, rank + rot a multiple of 32; RB >= rank / 16, KSM >= (rank + rot) / 32.
+// Sizes: rank and rot multiples of 32; RB >= rank / 16, KSM >= (rank + rot) / 32.
 typedef __bf16 la_bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 la_bf16x4 __attribute__((ext_vector_type(4)));
 typedef float la_f32x4 __attribute__((ext_vector_type(4)));
@@ -242,7 +243,8 @@ latent_attention_mfma_kernel(const float* __restrict__ q_full, const bf16* __res
     const bool head = h < H;
     const int pos = positions[t];
     const int* pt = page_table + (size_t)slots[seq_of[t]] * max_pages;
-    const int kd = rank + rot, KS = kd / 32, rblocks = rank / 16;
+    const int kd = rank + rot, KS = kd / 32, rblocks = rank / 16, vsteps = rank / 32;
+    __bf16* vt_w = Vt + (8 * g) * LA_VT_STRIDE + n;          // where this lane's numbers of a key go
 
     la_bf16x8 qh[KSM], ql[KSM];
     {
@@ -283,11 +285,14 @@ latent_attention_mfma_kernel(const float* __restrict__ q_full, const bf16* __res
                     s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kv, qh[ks], s[kb], 0, 0, 0);
                     s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kv, ql[ks], s[kb], 0, 0, 0);
                     // the same numbers are the key's part of V^T: key 16 kb + n, numbers 32 ks + 8 g + e
-                    if (32 * ks + 8 * g < rank) {
+                    if (ks < vsteps) {
 #pragma unroll
-                        for (int e = 0; e < 8; ++e) Vt[(32 * ks + 8 * g + e) * LA_VT_STRIDE + 16 * kb + n] = kv[e];
+                        for (int e = 0; e < 8; ++e) vt_w[(32 * ks + e) * LA_VT_STRIDE + 16 * kb] = kv[e];
                     }
                 }
+            // (the second block's loads stay behind the first block's products: all of a chunk's rows in
+            //  flight at once would not fit the registers beside the sums)
+            __builtin_amdgcn_sched_barrier(0);
         }
         // s[kb][i]: key j0 + 16 kb + 4 g + i against head n
         float cmax = -INFINITY;
@@ -317,6 +322,8 @@ latent_attention_mfma_kernel(const float* __restrict__ q_full, const bf16* __res
             }
         l = l * corr + psum;
         m = m_new;
+        // (rescaled every time: a branch around this, for chunks that leave the maximum as it is, made the
+        //  compiler spill the sums)
 #pragma unroll
         for (int db = 0; db < RB; ++db)
 #pragma unroll
@@ -326,10 +333,11 @@ latent_attention_mfma_kernel(const float* __restrict__ q_full, const bf16* __res
         for (int db = 0; db < RB; ++db)
             if (db < rblocks) {
                 const __bf16* vr = Vt + (db * 16 + n) * LA_VT_STRIDE + 4 * g;
-                const la_bf16x4 v0 = *(const la_bf16x4*)vr, v1 = *(const la_bf16x4*)(vr + 16);
-                const la_bf16x8 vv = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+                const uint2 v0 = *(const uint2*)vr, v1 = *(const uint2*)(vr + 16);
+                const la_bf16x8 vv = __builtin_bit_cast(la_bf16x8, uint4{v0.x, v0.y, v1.x, v1.y});
                 acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, ph, acc[db], 0, 0, 0);
                 acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, pl, acc[db], 0, 0, 0);
+                if (db % 8 == 7) __builtin_amdgcn_sched_barrier(0);      // (no more than eight blocks' reads in flight)
             }
         __syncthreads();
     }
@@ -388,8 +396,8 @@ extern "C" int hb_latent_attention_mfma(const float* q_full, const void* pages, 
                                         int page_size, int T, int H, int rank, int rot, float scale, int splits,
                                         int chunks_per_split, hipStream_t stream) {
     HB_REQUIRE(T > 0 && H > 0, "latent attention: empty input");
-    HB_REQUIRE(rank > 0 && rank % 16 == 0 && rank <= 512 && (rank + rot) % 32 == 0 && rank + rot <= 640,
-               "latent attention: the matrix-core kernel takes a latent in steps of 16 up to 512 whose row is a multiple of 32, not %d + %d", rank, rot);
+    HB_REQUIRE(rank > 0 && rank % 32 == 0 && rank <= 512 && rot % 32 == 0 && rank + rot <= 640,
+               "latent attention: the matrix-core kernel takes a latent and a rotated part in steps of 32, up to 512 + 128, not %d + %d", rank, rot);
     HB_REQUIRE(page_size % LA_CHUNK == 0, "latent attention: pages of %d positions", page_size);
     HB_REQUIRE(splits >= 1 && splits <= HB_WAVE && chunks_per_split >= 1, "latent attention: %d ranges, the kernels take 1 to 64", splits);
     HB_REQUIRE(splits == 1 || (part_acc && part_ml), "latent attention: ranges need scratch");

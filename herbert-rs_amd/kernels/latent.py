@@ -72,9 +72,9 @@ TARGET_WAVES = 1024        # a decode step's keys are cut into ranges until abou
 
 
 def mfma_takes(cache, rank, rot):
-    """True if the matrix-core kernel takes this latent: bfloat16 rows, rank in steps of 16 up to 512,
-    rows in steps of 32."""
-    return (cache.k.dtype == torch.bfloat16 and rank % 16 == 0 and 0 < rank <= 512 and (rank + rot) % 32 == 0
+    """True if the matrix-core kernel takes this latent: bfloat16 rows, the latent and the rotated part in
+    steps of 32, up to 512 + 128."""
+    return (cache.k.dtype == torch.bfloat16 and rank % 32 == 0 and 0 < rank <= 512 and rot % 32 == 0 and rot <= 128
             and cache.page_size % CHUNK == 0)
 
 
@@ -99,7 +99,7 @@ def latent_attention_mfma(q_full, meta, cache, out, gate, gate_off, H, rank, rot
         # the grid must not depend on the contexts themselves (a recorded step is replayed at others of its bucket)
         chunks = -(-max(meta.context_bucket, meta.max_context) // CHUNK)
         blocks = T * ((H + 15) // 16)
-        splits = max(1, min(TARGET_WAVES // blocks, -(-chunks // 4), 64))
+        splits = max(1, min(TARGET_WAVES // blocks, -(-chunks // 2), 64))
         per = -(-chunks // splits)
     part_acc = part_ml = None
     if splits > 1:

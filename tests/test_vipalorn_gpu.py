@@ -23,7 +23,7 @@ DTYPES = ["float32", "bfloat16"]
 # which no bound on rounding covers. Float32 is compared row by row without exception, and so is
 # bfloat16 where every expert is chosen (R); elsewhere a small share of the bfloat16 rows may be off,
 # and the rest must be as close as ever.
-FLIPPED_SHARE = 0.06
+FLIPPED_SHARE = {"S": 0.25}          # (twelve experts in four layers: more close calls, and the state carries one on)
 
 
 def compare(rows, folder, tokens, positions, dtype, label):
@@ -40,7 +40,7 @@ def compare(rows, folder, tokens, positions, dtype, label):
     if dtype == "float32" or every:
         assert not off, f"{label}: positions and errors {off[:5]}"
     else:
-        assert len(off) <= max(3, FLIPPED_SHARE * len(list(positions))), f"{label}: {len(off)} rows off: {off[:5]}"
+        assert len(off) <= max(3, FLIPPED_SHARE.get(name, 0.06) * len(list(positions))), f"{label}: {len(off)} rows off: {off[:5]}"
 
 
 def feed(engine, slot, tokens, cuts):
@@ -56,7 +56,7 @@ def feed(engine, slot, tokens, cuts):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["P", "Q", "R"])
+@pytest.mark.parametrize("name", ["P", "Q", "R", "S"])
 def test_whole_prompts_and_token_by_token(name, dtype, model_root):
     folder = make_folder(model_root, name, dtype)
     vocab = CONFIGS[name][0]["vocab"]
@@ -90,7 +90,7 @@ def test_portions_of_several_sizes_and_slots_used_again(name, dtype, model_root)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["P", "Q", "R"])
+@pytest.mark.parametrize("name", ["P", "Q", "R", "S"])
 def test_unequal_batches_against_each_alone(name, dtype, model_root):
     folder = make_folder(model_root, name, dtype)
     vocab = CONFIGS[name][0]["vocab"]

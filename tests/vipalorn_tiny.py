@@ -59,13 +59,21 @@ VIP_R = model(96, 64, [
     with_mlp(delta(1, 1, 48, 80, 1), None),
     with_mlp(latent(1, 16, 8, 16, 24, 0.5, base=100.0), moe(3, 3, 24, 0.75)),
 ], eps=1e-5, mult=1.0, logit_scale=1.0)
+# S: attention first and last around two delta layers, heads that share keys in pairs, three taps, a latent
+#    row that is no multiple of 32 (the plain attention kernel in either mode), three of twelve experts
+VIP_S = model(320, 192, [
+    with_mlp(latent(6, 24, 8, 40, 72, 0.2, base=40000.0), moe(12, 3, 80, 2.5)),
+    with_mlp(delta(4, 2, 40, 48, 3), moe(12, 3, 80, 2.5)),
+    with_mlp(delta(4, 2, 40, 48, 3), moe(12, 3, 80, 2.5)),
+    with_mlp(latent(6, 24, 8, 40, 72, 0.2, base=40000.0), moe(12, 3, 80, 2.5)),
+], eps=2e-5, mult=0.6, logit_scale=0.75)
 # W: the widths of a larger model's layers at a small depth: keys of 128 a head, a latent of 256 + 64
 VIP_W = model(1024, 512, [
     with_mlp(delta(8, 4, 128, 128, 4), moe(16, 4, 256, 7.0)),
     with_mlp(latent(8, 64, 64, 64, 256, 0.09), moe(16, 4, 256, 7.0)),
 ], eps=1e-6, mult=0.5, logit_scale=0.5)
 
-CONFIGS = {"P": (VIP_P, 11, 0.12), "Q": (VIP_Q, 12, 0.09), "R": (VIP_R, 13, 0.15), "W": (VIP_W, 14, 0.05)}
+CONFIGS = {"S": (VIP_S, 15, 0.08), "P": (VIP_P, 11, 0.12), "Q": (VIP_Q, 12, 0.09), "R": (VIP_R, 13, 0.15), "W": (VIP_W, 14, 0.05)}
 
 
 def make_folder(root, name, dtype="float32", scale=None, set_to=None, tag=""):
