@@ -290,6 +290,9 @@ extern "C" int hb_moe_combine(const float* y, const float* weight, const int* ro
 // The same products for bfloat16 operands with float32 sums (v_mfma_f32_16x16x32_bf16), and more
 // generally a group of products that share a shape: group g multiplies rows of A (from column
 // g * a_group_off on) with its own matrix W[g] [N, K] into columns of C from g * c_group_off on.
+// W[g] is stored in the order of the operands, [K / 32][N / 16][64 lanes][8] (the 1 KB of 16 rows and 32 k
+// in a row, lane = 16 (k / 8 % 4) + n % 16): a wave's load is one contiguous KB, where rows K apart
+// would each give 64 bytes from addresses a power of two apart.
 // The rows of a group come as a list of tiles (group, first row, rows <= 64) or, without a list, as
 // every group's ceil(M / 64) tiles of the same M rows (heads that each have a matrix of their own).
 // A workgroup is four waves on one tile of 64 rows; a wave holds four blocks of 16 weight rows
@@ -335,13 +338,15 @@ grouped_mfma_kernel(const bf16* __restrict__ A, int lda, size_t a_group_off, con
     // the wave's output columns: 64 of them, or with EPI 2 32 (from 32 gate rows and the 32 up rows that go with them)
     const int n0 = EPI == 2 ? (blockIdx.x * 4 + wave) * 32 : (blockIdx.x * 4 + wave) * 64;
     const bool idle = n0 >= out_cols;            // (such a wave still helps to load the activations)
+    // W[g] lies in the operands' order [K / 32][N / 16][64 lanes][8]: a block of 16 rows and 32 k is 1 KB in a row
     const bf16* Wg = W + (size_t)group * N * K;
+    const size_t kstep = (size_t)(N / 16) * 512;         // from a block to the same rows' next 32 k
     const bf16* wrow[4];
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
-        int n = (EPI == 2 ? (a < 2 ? n0 + 16 * a : F + n0 + 16 * (a - 2)) : n0 + 16 * a) + r16;
-        if (n >= N || idle) n = N - 1;               // (read a row that exists; its sums are not stored)
-        wrow[a] = Wg + (size_t)n * K + g4 * 8;
+        int nb = (EPI == 2 ? (a < 2 ? n0 + 16 * a : F + n0 + 16 * (a - 2)) : n0 + 16 * a) / 16;
+        if (nb >= N / 16 || idle) nb = N / 16 - 1;       // (read a block that exists; its sums are not stored)
+        wrow[a] = Wg + (size_t)nb * 512 + lane * 8;
     }
     const int blocks = (rows + 15) / 16;
     // what this thread brings of a stage: rows tid / 8 and 32 + tid / 8, piece tid % 8
@@ -370,7 +375,7 @@ grouped_mfma_kernel(const bf16* __restrict__ A, int lda, size_t a_group_off, con
         for (int h = 0; h < 2; ++h)
 #pragma unroll
             for (int a = 0; a < 4; ++a)
-                wnext[h][a] = k0 + 32 * h < K ? *(const hb_bf16x8*)(wrow[a] + k0 + 32 * h) : hb_bf16x8{};
+                wnext[h][a] = k0 + 32 * h < K ? *(const hb_bf16x8*)(wrow[a] + (size_t)(k0 / 32 + h) * kstep) : hb_bf16x8{};
     };
     fetch(0);
     for (int st = 0; st < stages; ++st) {
@@ -461,12 +466,13 @@ grouped_mfma_stream_kernel(const bf16* __restrict__ A, int lda, size_t a_group_o
     const int n0 = EPI == 2 ? (blockIdx.x * 4 + wave) * 16 : (blockIdx.x * 4 + wave) * 32;
     if (n0 >= out_cols) return;
     const bf16* Wg = W + (size_t)group * N * K;
+    const size_t kstep = (size_t)(N / 16) * 512;
     const bf16* wrow[2];
 #pragma unroll
     for (int a = 0; a < 2; ++a) {
-        int n = (EPI == 2 ? (a == 0 ? n0 : F + n0) : n0 + 16 * a) + r16;
-        if (n >= N) n = N - 1;                       // (read a row that exists; its sums are not stored)
-        wrow[a] = Wg + (size_t)n * K + g4 * 8;
+        int nb = (EPI == 2 ? (a == 0 ? n0 : F + n0) : n0 + 16 * a) / 16;
+        if (nb >= N / 16) nb = N / 16 - 1;           // (read a block that exists; its sums are not stored)
+        wrow[a] = Wg + (size_t)nb * 512 + lane * 8;
     }
     const int blocks = (rows + 15) / 16;
     const bf16* xrow[4];
@@ -487,7 +493,7 @@ grouped_mfma_stream_kernel(const bf16* __restrict__ A, int lda, size_t a_group_o
     for (int k = 0; k < K; k += 32) {
         hb_bf16x8 wv[2], xv[4];
 #pragma unroll
-        for (int a = 0; a < 2; ++a) wv[a] = *(const hb_bf16x8*)(wrow[a] + k);
+        for (int a = 0; a < 2; ++a) wv[a] = *(const hb_bf16x8*)(wrow[a] + (size_t)(k / 32) * kstep);
 #pragma unroll
         for (int b = 0; b < 4; ++b)
             if (b < blocks) xv[b] = *(const hb_bf16x8*)(xrow[b] + k);
@@ -539,6 +545,7 @@ extern "C" int hb_grouped_mfma(const void* A, int lda, size_t a_group_off, const
                                const int* tile_group, const int* tile_row0, const int* tile_rows, int n_tiles, int M,
                                int groups, float limit, float alpha, int few_rows, hipStream_t stream) {
     HB_REQUIRE(N > 0 && K > 0 && K % 32 == 0, "grouped product: K = %d must be a positive multiple of 32", K);
+    HB_REQUIRE(N % 16 == 0 && (epi != 2 || N % 32 == 0), "grouped product: %d weight rows are no whole blocks of 16", N);
     HB_REQUIRE(lda % 8 == 0 && a_group_off % 8 == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0,
                "grouped product: operands must lie at multiples of 16 bytes");
     HB_REQUIRE(epi >= 0 && epi <= 2 && (epi != 2 || N % 2 == 0), "grouped product: unknown epilogue %d", epi);

@@ -93,15 +93,25 @@ EPI_F32, EPI_BF16, EPI_GLU = 0, 1, 2
 FEW_ROWS = 16      # up to so many rows a group the kernel without a stage in LDS runs (decoding)
 
 
-def mfma_takes(K, lda, a_group_off=0):
-    """True if the matrix-core kernel takes products of this inner size and layout (bfloat16 operands)."""
-    return K % 32 == 0 and lda % 8 == 0 and a_group_off % 8 == 0
+def mfma_takes(K, lda, a_group_off=0, N=16):
+    """True if the matrix-core kernel takes products of this inner size, layout and N weight rows
+    (bfloat16 operands)."""
+    return K % 32 == 0 and lda % 8 == 0 and a_group_off % 8 == 0 and N % 16 == 0
+
+
+def pack_grouped(w):
+    """[G, N, K] -> the same values with every W[g] in the matrix cores' operand order [K / 32, N / 16, 64, 8]
+    (lane = 16 * (k / 8 % 4) + n % 16): what grouped_mfma reads."""
+    G, N, K = w.shape
+    if N % 16 or K % 32:
+        raise BackendError("packed matrices need N in steps of 16 and K in steps of 32")
+    return w.view(G, N // 16, 16, K // 32, 4, 8).permute(0, 3, 1, 4, 2, 5).contiguous().view(G, N, K)
 
 
 def grouped_mfma(a, lda, a_group_off, w, c, ldc, c_group_off, epi, routing=None, gather=False, M=0, limit=0.0,
                  alpha=0.0):
     """Group g: C[rows, g * c_group_off + n] = sum_k A[src(row), g * a_group_off + k] * w[g][n, k], bfloat16
-    operands, float32 sums. With `routing` the rows are the (token, expert) pairs in their experts' order
+    operands, float32 sums; w as pack_grouped gives it. With `routing` the rows are the (token, expert) pairs in their experts' order
     (gather: A's rows are the tokens'); without, every group takes the same M rows. epi: EPI_F32 / EPI_BF16
     store C in that type; EPI_GLU: w[g] is [2 F, K] (gate rows, then up rows) and C bfloat16 [*, F] receives
     the experts' activation with `limit` and `alpha`."""
@@ -109,7 +119,7 @@ def grouped_mfma(a, lda, a_group_off, w, c, ldc, c_group_off, epi, routing=None,
     _check(a, "a", torch.bfloat16)
     _check(w, "w", torch.bfloat16, (G, N, K))
     _check(c, "c", torch.bfloat16 if epi != EPI_F32 else torch.float32)
-    if not mfma_takes(K, lda, a_group_off):
+    if not mfma_takes(K, lda, a_group_off, N) or (epi == EPI_GLU and N % 32):
         raise BackendError(f"grouped product: K = {K}, rows {lda} apart and groups {a_group_off} apart are not taken")
     out_cols = N // 2 if epi == EPI_GLU else N
     if routing is not None:

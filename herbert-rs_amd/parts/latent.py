@@ -71,6 +71,11 @@ class LatentAttention(Part):
         self.uk_t = uk.transpose(1, 2).contiguous()
         self.uv = rt.weight(tensors[n["uv"]]).view(H, self.vdim, self.rank).contiguous()
         self.o = Linear(rt.weight(tensors[n["o"]]), scratch=rt.scratch)
+        # bfloat16 with sizes the matrix cores take: the heads' matrices are kept in their operands' order
+        self.cores = (rt.dtype == torch.bfloat16 and moe.mfma_takes(self.dim, H * self.dim, self.dim, self.rank)
+                      and moe.mfma_takes(self.rank, H * self.rank, self.rank, self.vdim))
+        if self.cores:
+            self.uk_t, self.uv = moe.pack_grouped(self.uk_t), moe.pack_grouped(self.uv)
         rot = self.position.rotation_rates()
         self.inv_freq, self.rot_dims = (None, 0) if rot is None else rot
         if self.rot_dims > self.rot_dim:
@@ -83,8 +88,7 @@ class LatentAttention(Part):
         proj = rt.buffer("latent_proj", (T, self.width), torch.float32)
         self.proj.forward(y, proj)
         q_full = rt.buffer("latent_q_full", (T, H * self.row), torch.float32)
-        cores = rt.dtype == torch.bfloat16 and moe.mfma_takes(self.dim, H * self.dim, self.dim) \
-            and moe.mfma_takes(self.rank, H * self.rank, self.rank)
+        cores = self.cores
         q_plain = rt.buffer("latent_q_plain", (T, H * self.dim), torch.bfloat16) if cores else None
         latent.latent_write(proj, 0, self.q_width, self.norm_w, q_full, self.inv_freq, ctx.meta, kv, H, self.dim,
                             self.rank, self.rot_dim, self.rot_dims, self.eps, write_cache=ctx.owns_cache,

@@ -56,6 +56,12 @@ class RoutedExperts(Part):
                                                rt.weight(tensors[n["up"].format(e=e)])], 0)
                                     for e in range(self.experts)]).contiguous()
         self.down = torch.stack([rt.weight(tensors[n["down"].format(e=e)]) for e in range(self.experts)]).contiguous()
+        # bfloat16 with sizes the matrix cores take: the matrices are kept in their operands' order
+        W, F = self.hidden_size, self.inter
+        self.cores = (rt.dtype == torch.bfloat16 and moe.mfma_takes(W, W, 0, 2 * F) and moe.mfma_takes(F, F, 0, W)
+                      and F % 16 == 0)
+        if self.cores:
+            self.gate_up, self.down = moe.pack_grouped(self.gate_up), moe.pack_grouped(self.down)
 
     def forward(self, ctx, y, x):
         rt = ctx.rt
@@ -67,7 +73,7 @@ class RoutedExperts(Part):
         moe.route(logits, self.router_bias, routing)
         act = rt.buffer("moe_act", (T * top, F))
         out = rt.buffer("moe_out", (T * top, self.hidden_size), torch.float32)
-        if y.dtype == torch.bfloat16 and moe.mfma_takes(self.hidden_size, self.hidden_size) and moe.mfma_takes(F, F):
+        if self.cores:
             # matrix cores; the activation is the first product's epilogue
             moe.grouped_mfma(y, self.hidden_size, 0, self.gate_up, act, F, 0, moe.EPI_GLU, routing, gather=True,
                              limit=self.limit, alpha=self.alpha)

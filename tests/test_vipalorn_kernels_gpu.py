@@ -255,8 +255,8 @@ def test_routing_groups_and_products(T, E, top):
         out = torch.empty(T * top, W, device=DEV)
         x = torch.zeros(T, W, device=DEV)
         if dtype == torch.bfloat16:
-            moe.grouped_mfma(yg, W, 0, gu_w, act, F, 0, moe.EPI_GLU, routing, gather=True, limit=1.5, alpha=1.702)
-            moe.grouped_mfma(act, F, 0, down_w, out, W, 0, moe.EPI_F32, routing)
+            moe.grouped_mfma(yg, W, 0, moe.pack_grouped(gu_w), act, F, 0, moe.EPI_GLU, routing, gather=True, limit=1.5, alpha=1.702)
+            moe.grouped_mfma(act, F, 0, moe.pack_grouped(down_w), out, W, 0, moe.EPI_F32, routing)
         else:
             gu = torch.empty(T * top, 2 * F, device=DEV)
             moe.gemm_plain(yg, gu_w, gu, routing, gather=True)
