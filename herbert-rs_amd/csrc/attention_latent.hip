@@ -368,24 +368,41 @@ latent_attention_mfma_kernel(const float* __restrict__ q_full, const bf16* __res
 }
 
 // out[row, :] = sum over the ranges (in order) of their sums, brought to one maximum, over the summed
-// denominators, times sigmoid(gate). One wave a (token, head).
-__global__ void __launch_bounds__(HB_WAVE)
+// denominators, times sigmoid(gate). One block a (token, head).
+__global__ void __launch_bounds__(256)
 latent_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml, bf16* __restrict__ out,
                     const float* __restrict__ gate, int gate_ld, int H, int rank, int splits) {
+    __shared__ float share[HB_WAVE + 1];          // the ranges' weights, and the row's factor
     const size_t row = blockIdx.x;
-    const int lane = threadIdx.x;
-    // lane s holds range s's share (at most 64 ranges)
-    const bool has = lane < splits;
-    const float ms = has ? part_ml[(row * splits + lane) * 2] : -INFINITY;
-    const float ls = has ? part_ml[(row * splits + lane) * 2 + 1] : 0.f;
-    const float m = hb_wave_max(ms);
-    const float ws = ms > -INFINITY ? expf(ms - m) : 0.f;
-    const float l = hb_wave_sum(ls * ws);
-    float w = l > 0.f ? 1.0f / l : 0.f;
-    if (gate) w *= 1.0f / (1.0f + expf(-gate[(row / H) * gate_ld + row % H]));
-    for (int d = lane; d < rank; d += HB_WAVE) {
+    if (threadIdx.x < HB_WAVE) {
+        // lane s holds range s's share (at most 64 ranges)
+        const int lane = threadIdx.x;
+        const bool has = lane < splits;
+        const float ms = has ? part_ml[(row * splits + lane) * 2] : -INFINITY;
+        const float ls = has ? part_ml[(row * splits + lane) * 2 + 1] : 0.f;
+        const float m = hb_wave_max(ms);
+        const float ws = ms > -INFINITY ? expf(ms - m) : 0.f;
+        const float l = hb_wave_sum(ls * ws);
+        float w = l > 0.f ? 1.0f / l : 0.f;
+        if (gate) w *= 1.0f / (1.0f + expf(-gate[(row / H) * gate_ld + row % H]));
+        share[lane] = ws;
+        if (lane == 0) share[HB_WAVE] = w;
+    }
+    __syncthreads();
+    const float w = share[HB_WAVE];
+    const float* pa = part_acc + row * splits * rank;
+    for (int d = threadIdx.x; d < rank; d += blockDim.x) {
         float a = 0.f;
-        for (int s = 0; s < splits; ++s) a = fmaf(part_acc[(row * splits + s) * rank + d], __shfl(ws, s, HB_WAVE), a);
+        int s2 = 0;
+        for (; s2 + 4 <= splits; s2 += 4) {            // (four ranges' loads at a time; summed in the ranges' order)
+            const float v0 = pa[(size_t)s2 * rank + d], v1 = pa[(size_t)(s2 + 1) * rank + d];
+            const float v2 = pa[(size_t)(s2 + 2) * rank + d], v3 = pa[(size_t)(s2 + 3) * rank + d];
+            a = fmaf(v0, share[s2], a);
+            a = fmaf(v1, share[s2 + 1], a);
+            a = fmaf(v2, share[s2 + 2], a);
+            a = fmaf(v3, share[s2 + 3], a);
+        }
+        for (; s2 < splits; ++s2) a = fmaf(pa[(size_t)s2 * rank + d], share[s2], a);
         out[row * rank + d] = hb_from_float<bf16>(a * w);
     }
 }
@@ -414,7 +431,7 @@ extern "C" int hb_latent_attention_mfma(const float* q_full, const void* pages, 
 #undef LA_LAUNCH
     HB_CHECK_LAUNCH("latent_attention_mfma");
     if (splits > 1) {
-        latent_merge_kernel<<<(unsigned)((long long)T * H), HB_WAVE, 0, stream>>>(part_acc, part_ml, (bf16*)out, gate, gate_ld, H, rank, splits);
+        latent_merge_kernel<<<(unsigned)((long long)T * H), 256, 0, stream>>>(part_acc, part_ml, (bf16*)out, gate, gate_ld, H, rank, splits);
         HB_CHECK_LAUNCH("latent_merge");
     }
     return 0;
