@@ -99,7 +99,7 @@ def latent_attention_mfma(q_full, meta, cache, out, gate, gate_off, H, rank, rot
         # the grid must not depend on the contexts themselves (a recorded step is replayed at others of its bucket)
         chunks = -(-max(meta.context_bucket, meta.max_context) // CHUNK)
         blocks = T * ((H + 15) // 16)
-        splits = max(1, min(TARGET_WAVES // blocks, -(-chunks // 2), 64))
+        splits = max(1, min(TARGET_WAVES // blocks, chunks, 64))
         per = -(-chunks // splits)
     part_acc = part_ml = None
     if splits > 1:
