@@ -102,14 +102,19 @@ extern "C" int hb_conv_silu(const float* proj, int ld, const float* taps, float*
 // fast as one token's step is short. A column is held by LPC lanes (each 16 of its D numbers, in
 // registers; LPC = 1 .. 16 for D up to 256), a wave holds 64 / LPC columns and walks the sequence's
 // tokens; a workgroup is one wave, so that a head's columns spread over many CUs. The two dot
-// products a token are summed over a column's lanes by exchanges within a row of 16 lanes. What a
+// products a token are summed over a column's lanes by exchanges within a row of 16 lanes (the first
+// runs on the numbers before their decay and is multiplied by g afterwards, g (S^T k) = (g S)^T k, so the
+// decay itself does not wait for it). What a
 // token needs (k, q, its values, g and beta, which do not wait for the chain) comes from a ring in
-// LDS that is filled 16 to 24 tokens ahead: a token's own loads would each cost the memory's latency.
+// LDS that is filled 16 to 32 tokens ahead: a token's own loads would each cost the memory's latency.
 // qkv rows: [kv_heads x D queries | kv_heads x D keys | heads x V values]; head h reads the
 // query and key of kv head h / (heads / kv_heads).
 #define DELTA_PER 16
-#define DELTA_SUB 8          // tokens that are loaded together
-#define DELTA_RING_OF(LPC) ((LPC) >= 16 ? 3 : 4)     // such groups in the ring (three where four would not fit 64 KB of LDS)
+// Tokens that are loaded together, and such groups in the ring. A group's loads are issued before the
+// group that is worked on and waited for after it, so a group must take longer than the memory's latency:
+// with 8 tokens a group the kernel took that latency over 8 a token. (8 where 16 would not fit 64 KB of LDS.)
+#define DELTA_SUB_OF(LPC) ((LPC) >= 16 ? 8 : 16)
+#define DELTA_RING_OF(LPC) 3
 
 __device__ __forceinline__ float delta_dpp(float v, const int ctrl) {
     // (a lane reads another lane's value: ctrl names which, within rows of 16 lanes)
@@ -141,6 +146,7 @@ gated_delta_kernel(const float* __restrict__ qkv, int C, const float* __restrict
     constexpr int COLS = HB_WAVE / LPC;
     constexpr int DP = LPC * DELTA_PER;                 // D rounded up to what the lanes hold
     constexpr int DELTA_RING = DELTA_RING_OF(LPC);
+    constexpr int DELTA_SUB = DELTA_SUB_OF(LPC);
     constexpr int SLOTS = DELTA_SUB * DELTA_RING;
     constexpr int KQ4 = DELTA_SUB * DP / 2;             // float4 of k and q a group of tokens
     constexpr int KQ_PER_LANE = (KQ4 + HB_WAVE - 1) / HB_WAVE;
@@ -247,21 +253,20 @@ gated_delta_kernel(const float* __restrict__ qkv, int C, const float* __restrict
             }
             const float vc = v_ring[s0 + i][lcol];
             const float g = gb_ring[s0 + i][0], beta = gb_ring[s0 + i][1];
-            float dot = 0.f;
+            // g (S^T k) = (g S)^T k: the dot product runs on the old numbers, in four partial sums, and the
+            // decay of the numbers themselves does not wait for it
+            float d4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int e = 0; e < DELTA_PER; ++e) {
-                S[e] *= g;
-                dot = fmaf(S[e], kc[e], dot);
-            }
-            dot = delta_column_sum<LPC>(dot);
+            for (int e = 0; e < DELTA_PER; ++e) d4[e & 3] = fmaf(S[e], kc[e], d4[e & 3]);
+            const float dot = g * delta_column_sum<LPC>((d4[0] + d4[1]) + (d4[2] + d4[3]));
             const float u = beta * (vc - dot);
-            float o = 0.f;
+            float o4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int e = 0; e < DELTA_PER; ++e) {
-                S[e] = fmaf(kc[e], u, S[e]);
-                o = fmaf(S[e], qc[e], o);
+                S[e] = fmaf(kc[e], u, g * S[e]);
+                o4[e & 3] = fmaf(S[e], qc[e], o4[e & 3]);
             }
-            o = delta_column_sum<LPC>(o);
+            const float o = delta_column_sum<LPC>((o4[0] + o4[1]) + (o4[2] + o4[3]));
             if (live && part == 0) out[(size_t)(t0 + i) * heads * V + h * V + col] = o;
         }
         if (ahead) stash(p + DELTA_RING - 1);           // (the place of the group before this one)
