@@ -1,6 +1,6 @@
 // A feed-forward of many small experts of which each token uses a few.
 //   route     the router's logits (+ bias) of a token -> its `top` experts (largest logits, the
-//             lower index of equals) and their weights, the softmax over the chosen logits only
+//             lower index of equals), weighed by exp(logit) normalised over those experts alone
 //   group     the (token, choice) pairs in the order of their experts, so that an expert's rows
 //             are consecutive, and a list of row tiles (expert, first row, rows) of fixed length
 //   products  a tile's rows times its expert's matrix, float32 sums over k ascending by one

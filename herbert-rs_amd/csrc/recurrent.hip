@@ -1,5 +1,5 @@
 // Kernels of mixers that carry a state of fixed size from token to token instead of keys and
-// values: a short causal convolution over time per channel (its last inputs are state), and the
+// values: a filter of a few taps along time, channel by channel (its last inputs are state), and the
 // gated delta rule, a matrix of state a head that every token first decays, then corrects towards
 // its value along its key, then reads with its query. Everything here is float32.
 //

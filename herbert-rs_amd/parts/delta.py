@@ -1,8 +1,8 @@
 """A mixer with a matrix of state a head instead of keys and values: the gated delta rule.
 
-From the normed rows h:  q = W_q h, k = W_k h (kv_heads x dim), v = W_v h (heads x vdim), each through a
-short causal convolution over time per channel (taps [channels, K], the last column the current
-token's, zeros before the sequence's start) and silu; q and k then unit vectors a head
+From the normed rows h:  q = W_q h, k = W_k h (kv_heads x dim), v = W_v h (heads x vdim), each filtered
+along time, channel by channel, over the token and the K - 1 tokens before it (taps [channels, K], column
+K - 1 weighs the token itself; nothing precedes a sequence's first token) and then through silu; q and k then unit vectors a head
 (x / sqrt(sum x^2 + 1e-6)), q times dim^-1/2. A head h (on q/k head h / (heads / kv_heads)) keeps
 S [dim, vdim], zero at the start, and for every token
     S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q

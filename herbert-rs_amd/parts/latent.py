@@ -6,8 +6,8 @@ are one key part that all heads share. Head n's key is [W_uk,n c | that part], i
 score is the dot product of query and key times `scale`, causal, plain softmax; the head's output is
 multiplied by sigmoid(W_g h)_n and the heads go through W_o.
 
-Only c and the rotated part are cached, one row a token ([kv_rank + rot_dim], no values of their
-own). The kernels never build a head's keys or values: the query's unrotated part is taken through
+What a token leaves in the cache is c and the rotated part, one row of kv_rank + rot_dim numbers, and
+no values beside them. The kernels never build a head's keys or values: the query's unrotated part is taken through
 W_uk,n^T first (kv_rank numbers), scores and weighted sums then run on the cached rows themselves,
 one shared "key head" for all query heads, and the summed latents go through W_uv,n afterwards.
 Scores, softmax and the weighted sums are float32 in either mode.

@@ -1,7 +1,7 @@
 """A feed-forward of many small experts, of which each token uses a few.
 
-Router: z = W_r y + b in float32; the `top` experts with the largest z are chosen, and their weights
-are the softmax over the chosen z only. An expert: g = min(W_gate y, limit), u = clamp(W_up y, -limit,
+Router: z = W_r y + b in float32. A token goes to the `top` experts whose z is largest, and weighs them by
+exp(z) normalised over those experts alone (not over all of them). An expert: g = min(W_gate y, limit), u = clamp(W_up y, -limit,
 limit), out = W_down (g sigmoid(alpha g) (u + 1)), no biases. The part's output is the weighted sum
 of the chosen experts' outputs. The routing never reaches the host: the (token, expert) pairs are put
 in the order of their experts on the GPU and the experts' products run over a list of row tiles of

@@ -52,8 +52,8 @@ def softplus(x):
 
 # ---------------------------------------------------------------- short convolution
 def short_conv(x, taps):
-    """y[t, c] = sum_j taps[c, j] * x[t - (K - 1) + j, c], zeros before the start; the last
-    column of `taps` weighs the current token. x [T, C], taps [C, K]."""
+    """y[t, c] = sum_j taps[c, j] * x[t - (K - 1) + j, c] with x = 0 at negative times, so taps[:, K - 1]
+    belongs to token t itself. x [T, C], taps [C, K]."""
     T, C = x.shape
     K = taps.shape[1]
     out = torch.zeros_like(x)
@@ -109,7 +109,7 @@ def delta_mixer(h, w, p, mixer, eps):
 def rotate_half_layout(x, positions, base, dims):
     """The first `dims` entries of the last axis rotated: entry i pairs with i + dims/2; the pair
     (a, b) at position p becomes (a cos - b sin, b cos + a sin), angle p * base^(-2i/dims).
-    x [T, ..., n >= dims]; the rest passes unchanged."""
+    x [T, ..., n >= dims]; entries from `dims` on are copied."""
     half = dims // 2
     i = torch.arange(half, dtype=x.dtype)
     freq = torch.as_tensor(base, dtype=x.dtype) ** (-2.0 * i / dims)
@@ -122,8 +122,8 @@ def rotate_half_layout(x, positions, base, dims):
 
 # ---------------------------------------------------------------- latent attention
 def latent_attention_mixer(h, positions, w, p, mixer, eps):
-    """Keys and values of every head come from one latent c a token (and one rotated key part
-    shared by the heads); causal softmax attention; a sigmoid gate a head on the output."""
+    """Attention with the heads' own keys [W_uk c | r] and values W_uv c built from a token's latent c and the
+    rotated part r that all heads use; causal softmax; every head's output times a sigmoid gate."""
     H, D, R, V, rank = mixer["heads"], mixer["dim"], mixer["rot_dim"], mixer["vdim"], mixer["kv_rank"]
     rot = mixer["rot"]
     T = h.shape[0]

@@ -67,7 +67,7 @@ def test_whole_prompts_and_token_by_token(name, dtype, model_root):
         compare(feed(engine, slot, tokens, []), folder, tokens, range(n), dtype, f"{name} whole")
         engine.free_slot(slot)
     # the first tokens of a sequence one by one, then on through a page's edge: the state of a fresh slot,
-    # the convolution's zeros before the start, the first keys
+    # the filter's empty past, the first keys
     tokens = random_tokens(vocab, 70, 5)
     slot = engine.alloc_slot()
     compare(feed(engine, slot, tokens, range(1, 70)), folder, tokens, range(70), dtype, f"{name} one by one")

@@ -39,7 +39,7 @@ def test_delta_rule_special_cases():
     # no decay, full step, orthonormal keys: token t's value is stored along its key and read back exactly
     eye = torch.eye(D, dtype=torch.float64)[[0, 1, 2, 3, 0, 1]]
     out = plain.delta_rule(eye, eye, v, ones, ones)
-    assert torch.allclose(out, v, atol=1e-12)                  # the read-out sees the token's own write
+    assert torch.allclose(out, v, atol=1e-12)                  # o_t is read after token t has been written
     # beta 0 writes nothing: the state stays zero
     assert torch.equal(plain.delta_rule(q, k, v, zeros, ones), torch.zeros(T, V, dtype=torch.float64))
     # decay 0 forgets everything before the token: o_t = beta (k_t . q_t) v_t
