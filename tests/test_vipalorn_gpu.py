@@ -200,6 +200,28 @@ def test_the_trace_program(dtype, model_root, tmp_path):
             compare([row], folder, reqs[rid], [pos], dtype, f"P trace {label}")
 
 
+def test_the_command_line_generates_token_ids(model_root):
+    """The command line serves the family as it serves any other: token ids in, token ids out (--max-tokens 6 gives
+    seven tokens: it counts the decode steps after the prompt's own token), with sampling parameters too."""
+    import os
+    import subprocess
+    import sys
+    folder = make_folder(model_root, "P", "float32")
+    cfg, w = plain_folder(folder)
+    cli = os.path.join(ru.ROOT, "bin", "herbert-cli")
+    out = subprocess.run([sys.executable, cli, "--model", folder, "--prompt", "5,17,3,190", "--temperature", "0",
+                          "--max-tokens", "6", "--dtype", "float32", "--ignore-eos", "--no-repeat-check", "--verbose"],
+                         capture_output=True, text=True, timeout=240)
+    assert out.returncode == 0, out.stderr
+    assert [int(t) for t in out.stdout.strip().split(",")] == plain.greedy(cfg, w, [5, 17, 3, 190], 7)
+    drawn = [subprocess.run([sys.executable, cli, "--model", folder, "--prompt", "5,17,3,190", "--temperature", "0.8",
+                             "--top-k", "20", "--top-p", "0.9", "--seed", "3", "--max-tokens", "6", "--dtype", "float32",
+                             "--ignore-eos", "--no-repeat-check"], capture_output=True, text=True, timeout=240)
+             for _ in range(2)]
+    assert all(d.returncode == 0 for d in drawn), drawn[0].stderr
+    assert drawn[0].stdout == drawn[1].stdout and len(drawn[0].stdout.strip().split(",")) == 7
+
+
 def test_configuration_errors_and_the_registry(model_root):
     from herbert_rs_amd.config import load_config
     from herbert_rs_amd.errors import ConfigError
