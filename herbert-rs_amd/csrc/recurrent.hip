@@ -99,7 +99,7 @@ extern "C" int hb_conv_silu(const float* proj, int ld, const float* taps, float*
 //   S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q        (o sees the token's own write)
 // with g = exp(-exp(A_log[h]) * softplus(a + dt_bias[h])) and beta = sigmoid(b), a and b columns of
 // the projection's row. The columns of S never meet, and the tokens are a chain: the kernel is as
-// fast as one token's step is short. A column is held by LPC lanes (each 16 of its D numbers, in
+// fast as one token's step is short. A column is held by LPC lanes (each 8 or 16 of its D numbers, in
 // registers; LPC = 1 .. 16 for D up to 256), a wave holds 64 / LPC columns and walks the sequence's
 // tokens; a workgroup is one wave, so that a head's columns spread over many CUs. The two dot
 // products a token are summed over a column's lanes by exchanges within a row of 16 lanes (the first
@@ -109,11 +109,10 @@ extern "C" int hb_conv_silu(const float* proj, int ld, const float* taps, float*
 // LDS that is filled 16 to 32 tokens ahead: a token's own loads would each cost the memory's latency.
 // qkv rows: [kv_heads x D queries | kv_heads x D keys | heads x V values]; head h reads the
 // query and key of kv head h / (heads / kv_heads).
-#define DELTA_PER 16
 // Tokens that are loaded together, and such groups in the ring. A group's loads are issued before the
 // group that is worked on and waited for after it, so a group must take longer than the memory's latency:
 // with 8 tokens a group the kernel took that latency over 8 a token. (8 where 16 would not fit 64 KB of LDS.)
-#define DELTA_SUB_OF(LPC) ((LPC) >= 16 ? 8 : 16)
+#define DELTA_SUB_OF(DP) ((DP) >= 256 ? 8 : 16)
 #define DELTA_RING_OF(LPC) 3
 
 __device__ __forceinline__ float delta_dpp(float v, const int ctrl) {
@@ -137,7 +136,7 @@ __device__ __forceinline__ float delta_column_sum(float v) {
     return v;
 }
 
-template <int LPC>
+template <int LPC, int DELTA_PER>
 __global__ void __launch_bounds__(HB_WAVE)
 gated_delta_kernel(const float* __restrict__ qkv, int C, const float* __restrict__ proj, int ld, int b_off,
                    int a_off, const float* __restrict__ A_log, const float* __restrict__ dt_bias,
@@ -146,7 +145,7 @@ gated_delta_kernel(const float* __restrict__ qkv, int C, const float* __restrict
     constexpr int COLS = HB_WAVE / LPC;
     constexpr int DP = LPC * DELTA_PER;                 // D rounded up to what the lanes hold
     constexpr int DELTA_RING = DELTA_RING_OF(LPC);
-    constexpr int DELTA_SUB = DELTA_SUB_OF(LPC);
+    constexpr int DELTA_SUB = DELTA_SUB_OF(LPC * DELTA_PER);
     constexpr int SLOTS = DELTA_SUB * DELTA_RING;
     constexpr int KQ4 = DELTA_SUB * DP / 2;             // float4 of k and q a group of tokens
     constexpr int KQ_PER_LANE = (KQ4 + HB_WAVE - 1) / HB_WAVE;
@@ -156,7 +155,7 @@ gated_delta_kernel(const float* __restrict__ qkv, int C, const float* __restrict
     __shared__ float gb_ring[SLOTS][2];
     const int seq = blockIdx.x, h = blockIdx.y;
     const int lane = threadIdx.x;
-    const int part = lane % LPC;                       // which 16 of the column's D numbers
+    const int part = lane % LPC;                       // which of the column's D numbers this lane holds
     const int lcol = lane / LPC;
     const int col0 = blockIdx.z * COLS;
     const int col = col0 + lcol;
@@ -287,17 +286,32 @@ extern "C" int hb_gated_delta(const float* qkv, int C, const float* proj, int ld
     HB_REQUIRE(D > 0 && D <= 256, "delta rule: keys of %d, the kernel takes 1 to 256", D);
     HB_REQUIRE(V > 0 && C == 2 * kv_heads * D + heads * V, "delta rule: %d channels do not fit the heads", C);
     HB_REQUIRE(B <= 65535 && heads <= 65535, "delta rule: too many sequences or heads for the grid");
-    const int lpc = D <= 16 ? 1 : D <= 32 ? 2 : D <= 64 ? 4 : D <= 128 ? 8 : 16;
+    // Lanes a column x numbers a lane. Few waves (one prompt): 8 numbers a lane, so that a token's step is
+    // short (the chain is what counts: 2,048 tokens of 16 heads of 128 x 128 take 0.97 ms with 16 numbers a
+    // lane and 0.77 ms with 8). Many waves (a batch): 16 numbers a lane, half the waves and fewer
+    // instructions in all (a decode step of 8 sequences: 15 us against 30).
+    const int narrow = D <= 16 ? 1 : D <= 32 ? 2 : D <= 64 ? 4 : D <= 128 ? 8 : 16;        // lanes a column with 16 numbers a lane
+    const long long waves = (long long)B * heads * ((V + HB_WAVE / narrow - 1) / (HB_WAVE / narrow));
+    const bool wide = D <= 128 && (D <= 8 || waves <= 512);
+    const int lpc = wide ? (D <= 8 ? 1 : D <= 16 ? 2 : D <= 32 ? 4 : D <= 64 ? 8 : 16) : narrow;
     const int cols = HB_WAVE / lpc;
     const dim3 grid(B, heads, (V + cols - 1) / cols);
-#define HB_DELTA(L)                                                                                               \
-    gated_delta_kernel<L><<<grid, HB_WAVE, 0, stream>>>(qkv, C, proj, ld, b_off, a_off, A_log, dt_bias, state,     \
-                                                        seq_starts, slots, out, kv_heads, heads, D, V)
-    if (lpc == 1) HB_DELTA(1);
-    else if (lpc == 2) HB_DELTA(2);
-    else if (lpc == 4) HB_DELTA(4);
-    else if (lpc == 8) HB_DELTA(8);
-    else HB_DELTA(16);
+#define HB_DELTA(L, P)                                                                                            \
+    gated_delta_kernel<L, P><<<grid, HB_WAVE, 0, stream>>>(qkv, C, proj, ld, b_off, a_off, A_log, dt_bias, state,  \
+                                                           seq_starts, slots, out, kv_heads, heads, D, V)
+    if (wide) {
+        if (lpc == 1) HB_DELTA(1, 8);
+        else if (lpc == 2) HB_DELTA(2, 8);
+        else if (lpc == 4) HB_DELTA(4, 8);
+        else if (lpc == 8) HB_DELTA(8, 8);
+        else HB_DELTA(16, 8);
+    } else {
+        if (lpc == 1) HB_DELTA(1, 16);
+        else if (lpc == 2) HB_DELTA(2, 16);
+        else if (lpc == 4) HB_DELTA(4, 16);
+        else if (lpc == 8) HB_DELTA(8, 16);
+        else HB_DELTA(16, 16);
+    }
 #undef HB_DELTA
     HB_CHECK_LAUNCH("gated_delta");
     return 0;
