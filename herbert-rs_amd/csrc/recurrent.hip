@@ -286,13 +286,13 @@ extern "C" int hb_gated_delta(const float* qkv, int C, const float* proj, int ld
     HB_REQUIRE(D > 0 && D <= 256, "delta rule: keys of %d, the kernel takes 1 to 256", D);
     HB_REQUIRE(V > 0 && C == 2 * kv_heads * D + heads * V, "delta rule: %d channels do not fit the heads", C);
     HB_REQUIRE(B <= 65535 && heads <= 65535, "delta rule: too many sequences or heads for the grid");
-    // Lanes a column x numbers a lane. Few waves (one prompt): 8 numbers a lane, so that a token's step is
+    // Lanes a column x numbers a lane. Few waves (one prompt of a model of up to 16 heads of 128 columns): 8 numbers a lane, so that a token's step is
     // short (the chain is what counts: 2,048 tokens of 16 heads of 128 x 128 take 0.97 ms with 16 numbers a
     // lane and 0.77 ms with 8). Many waves (a batch): 16 numbers a lane, half the waves and fewer
     // instructions in all (a decode step of 8 sequences: 15 us against 30).
     const int narrow = D <= 16 ? 1 : D <= 32 ? 2 : D <= 64 ? 4 : D <= 128 ? 8 : 16;        // lanes a column with 16 numbers a lane
     const long long waves = (long long)B * heads * ((V + HB_WAVE / narrow - 1) / (HB_WAVE / narrow));
-    const bool wide = D <= 128 && (D <= 8 || waves <= 512);
+    const bool wide = D <= 128 && (D <= 8 || waves <= 256);        // (twice as many must still run at once: three a CU by their LDS)
     const int lpc = wide ? (D <= 8 ? 1 : D <= 16 ? 2 : D <= 32 ? 4 : D <= 64 ? 8 : 16) : narrow;
     const int cols = HB_WAVE / lpc;
     const dim3 grid(B, heads, (V + cols - 1) / cols);
