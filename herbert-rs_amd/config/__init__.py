@@ -4,6 +4,7 @@ from .registry import (Architecture, ChatFormat, load_config, register_architect
                        registered_architectures, resolve_architecture)
 from .qwen3 import Qwen3Config
 from .vipalorn import VipalornConfig
+from .modasun import ModasunConfig
 
-__all__ = ["Architecture", "ChatFormat", "Qwen3Config", "VipalornConfig", "load_config", "read_config_json",
+__all__ = ["Architecture", "ChatFormat", "ModasunConfig", "Qwen3Config", "VipalornConfig", "load_config", "read_config_json",
            "register_architecture", "registered_architectures", "resolve_architecture"]

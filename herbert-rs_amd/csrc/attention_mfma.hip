@@ -639,6 +639,9 @@ struct DecodeFusion {
     float eps;
     int write_kv;
     size_t slice_stride;
+    // a query at position p is multiplied by 1 + q_temp_coef * ln(floor((p + 1) / q_temp_every) + 1); every <= 0: by 1
+    float q_temp_coef;
+    int q_temp_every;
 };
 
 template <int HD, bool FUSED, int QS = 1>
@@ -796,6 +799,8 @@ attn_decode_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_cache, bf16*
             }
             __threadfence_block();      // this wave's later loads of that page see what it has just written
         }
+        const float grow = fu.q_temp_every > 0
+                               ? 1.0f + fu.q_temp_coef * logf((float)((hi + 1) / fu.q_temp_every) + 1.0f) : 1.0f;
         auto finish_head = [&](int hl, float x0, float x1) {
             if (fu.q_norm_w) {
                 float ss = x0 * x0 + x1 * x1;
@@ -805,6 +810,8 @@ attn_decode_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_cache, bf16*
                 x0 = x0 * inv * qw0;
                 x1 = x1 * inv * qw1;
             }
+            x0 *= grow;
+            x1 *= grow;
             if (hl < G) {
                 qs[hl * HD + j] = hb_from_float<bf16>(x0 * cs - x1 * sn);
                 qs[hl * HD + j + HALF] = hb_from_float<bf16>(x0 * sn + x1 * cs);
@@ -1045,7 +1052,7 @@ extern "C" int hb_attn_decode_mfma(const void* q, void* k_cache, void* v_cache, 
                                    int pages_per_split, const float* qkv, const float* q_norm_w,
                                    const float* k_norm_w, const float* cos_t, const float* sin_t, float eps,
                                    int write_kv, int qkv_slices, size_t slice_stride, const int* ranges,
-                                   hipStream_t stream) {
+                                   float q_temp_coef, int q_temp_every, hipStream_t stream) {
     // ranges != null: see attn_decode_kernel; `splits` is then the number of items of the grid (the
     // partial results are [nq, splits]), pages_per_split is not read
     HB_REQUIRE(!ranges || (B >= 2 && splits >= 2 && window == 0),
@@ -1061,7 +1068,7 @@ extern "C" int hb_attn_decode_mfma(const void* q, void* k_cache, void* v_cache, 
                "attn_decode: %d slices of the projection are not taken here", qkv_slices);
     dim3 grid(ranges ? 1 : B, nkv, splits);
     const float c = scale * LOG2E;
-    const DecodeFusion fu = {qkv, q_norm_w, k_norm_w, cos_t, sin_t, eps, write_kv, slice_stride};
+    const DecodeFusion fu = {qkv, q_norm_w, k_norm_w, cos_t, sin_t, eps, write_kv, slice_stride, q_temp_coef, q_temp_every};
     bf16* const direct = splits == 1 ? (bf16*)out : nullptr;      // one range: the kernel writes the output itself
     HB_REQUIRE(qkv || q, "attn_decode: neither q nor the projection rows are given");
     HB_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "attn_decode: cos and sin tables come together");

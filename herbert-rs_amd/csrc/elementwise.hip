@@ -166,6 +166,12 @@ extern "C" int hb_rmsnorm(const float* x, const float* w, void* y, int y_dtype, 
     return 0;
 }
 
+// A query's factor at position p: 1 + coef * ln(floor((p + 1) / every) + 1); every <= 0: none.
+__device__ __forceinline__ float hb_query_temperature(int pos, float coef, int every) {
+    if (every <= 0) return 1.0f;
+    return 1.0f + coef * logf((float)((pos + 1) / every) + 1.0f);
+}
+
 // ------------------------------------- per-head norm + rotation + cache write
 // One wave per (token, head) of the fused projection row [q heads | k heads | v heads].
 //   q heads: optional RMSNorm over the head, optional rotation, written to q_out.
@@ -182,7 +188,7 @@ __global__ void qk_norm_rope_write_kernel(
     int rot_dims, const int* __restrict__ positions, const int* __restrict__ seq_of,
     const int* __restrict__ slots, const int* __restrict__ page_table, int max_pages, int page_size,
     TQ* __restrict__ q_out, TC* __restrict__ k_cache, TC* __restrict__ v_cache, int nq, int nkv, int hd,
-    float eps) {
+    float eps, float q_temp_coef, int q_temp_every) {
     __shared__ float vec[HB_MAX_HEAD_DIM];
     const int t = blockIdx.x;
     const int h = blockIdx.y;
@@ -206,6 +212,8 @@ __global__ void qk_norm_rope_write_kernel(
     const bool do_rope = !is_v && cos_t != nullptr;
     const float inv = do_norm ? 1.0f / sqrtf(ss / (float)hd + eps) : 1.0f;
     const int half = rot_dims / 2;
+    // a query may grow with its position (see hb_query_temperature)
+    const float grow = is_q ? hb_query_temperature(pos, q_temp_coef, q_temp_every) : 1.0f;
 
     size_t dst_base = 0;      // keys: start of the token's row; values: start of the (page, head) block
     if (!is_q) {
@@ -234,7 +242,7 @@ __global__ void qk_norm_rope_write_kernel(
             if (do_norm) out = out * inv * norm_w[d];
         }
         if (is_q)
-            q_out[(size_t)t * nq * hd + (size_t)h * hd + d] = hb_from_float<TQ>(out);
+            q_out[(size_t)t * nq * hd + (size_t)h * hd + d] = hb_from_float<TQ>(out * grow);
         else if (is_v)
             v_cache[dst_base + (size_t)d * page_size + in_page] = hb_from_float<TC>(out);
         else
@@ -256,7 +264,8 @@ __global__ void __launch_bounds__(256) qk_norm_rope_write_tiled_kernel(
     const float* __restrict__ k_norm_w, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
     const int* __restrict__ positions, const int* __restrict__ seq_of, const int* __restrict__ slots,
     const int* __restrict__ page_table, int max_pages, int page_size, TQ* __restrict__ q_out,
-    TC* __restrict__ k_cache, TC* __restrict__ v_cache, int T, int nq, int nkv, int hd, float eps) {
+    TC* __restrict__ k_cache, TC* __restrict__ v_cache, int T, int nq, int nkv, int hd, float eps,
+    float q_temp_coef, int q_temp_every) {
     __shared__ float vt[64][HB_TILED_HEAD_DIM + 1];
     const int t0 = blockIdx.x * 64, h = blockIdx.y;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -347,6 +356,11 @@ __global__ void __launch_bounds__(256) qk_norm_rope_write_tiled_kernel(
                 a = o;
             }
             if (!mine || t >= T) continue;
+            if (is_q && q_temp_every > 0) {
+                const float grow = hb_query_temperature(pos[u], q_temp_coef, q_temp_every);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) a[e] *= grow;
+            }
             TQ packed[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) packed[e] = hb_from_float<TQ>(a[e]);
@@ -367,7 +381,8 @@ extern "C" int hb_qk_norm_rope_write(const float* qkv, int ld_qkv, const float* 
                                      const int* slots, const int* page_table, int max_pages,
                                      int page_size, void* q_out, void* k_cache, void* v_cache, int dtype,
                                      int T, int nq, int nkv, int hd, float eps, int write_kv,
-                                     int qkv_slices, size_t slice_stride, hipStream_t stream) {
+                                     int qkv_slices, size_t slice_stride, float q_temp_coef, int q_temp_every,
+                                     hipStream_t stream) {
     HB_REQUIRE(T > 0 && nq > 0 && nkv > 0, "qk_norm_rope_write: empty input");
     HB_REQUIRE(hd > 0 && hd <= HB_MAX_HEAD_DIM, "qk_norm_rope_write: head_dim %d not in 1..%d", hd,
                HB_MAX_HEAD_DIM);
@@ -385,7 +400,8 @@ extern "C" int hb_qk_norm_rope_write(const float* qkv, int ld_qkv, const float* 
 #define TILED_GO(QSV)                                                                                          \
     qk_norm_rope_write_tiled_kernel<bf16, bf16, QSV><<<tiles, 256, 0, stream>>>(                              \
         qkv, ld_qkv, slice_stride, q_norm_w, k_norm_w, cos_t, sin_t, positions, seq_of, slots, page_table,    \
-        max_pages, page_size, (bf16*)q_out, (bf16*)k_cache, (bf16*)v_cache, T, nq, nkv, hd, eps)
+        max_pages, page_size, (bf16*)q_out, (bf16*)k_cache, (bf16*)v_cache, T, nq, nkv, hd, eps, q_temp_coef,   \
+        q_temp_every)
         if (qkv_slices == 1) TILED_GO(1);
         else if (qkv_slices == 2) TILED_GO(2);
         else if (qkv_slices == 4) TILED_GO(4);
@@ -401,12 +417,12 @@ extern "C" int hb_qk_norm_rope_write(const float* qkv, int ld_qkv, const float* 
         qk_norm_rope_write_kernel<float, float><<<grid, HB_WAVE, 0, stream>>>(
             qkv, ld_qkv, q_norm_w, k_norm_w, cos_t, sin_t, rot_dims, positions, seq_of, slots,
             page_table, max_pages, page_size, (float*)q_out, (float*)k_cache, (float*)v_cache, nq, nkv,
-            hd, eps);
+            hd, eps, q_temp_coef, q_temp_every);
     else if (dtype == HB_BF16)
         qk_norm_rope_write_kernel<bf16, bf16><<<grid, HB_WAVE, 0, stream>>>(
             qkv, ld_qkv, q_norm_w, k_norm_w, cos_t, sin_t, rot_dims, positions, seq_of, slots,
             page_table, max_pages, page_size, (bf16*)q_out, (bf16*)k_cache, (bf16*)v_cache, nq, nkv, hd,
-            eps);
+            eps, q_temp_coef, q_temp_every);
     else
         HB_REQUIRE(false, "qk_norm_rope_write: unknown dtype %d", dtype);
     HB_CHECK_LAUNCH("qk_norm_rope_write");
@@ -526,5 +542,74 @@ extern "C" int hb_scale(float* x, float s, size_t n, hipStream_t stream) {
     const size_t blocks = (n + 255) / 256;
     scale_kernel<<<(unsigned)(blocks > 4096 ? 4096 : blocks), 256, 0, stream>>>(x, s, n);
     HB_CHECK_LAUNCH("scale");
+    return 0;
+}
+
+// ------------------------------------------------- a layer whose norm comes after the sum
+// Between two parts of such a layer the stream is x <- norm(alpha x + part(x)). The parts add their
+// outputs to rows that already hold alpha x; this kernel then makes from such rows `src`, a row a block,
+//   x = src / sqrt(mean(src^2) + eps) * w      (w null: x = src, the stream's first rows)
+//   y = x in the compute dtype                 (what the next part reads; null: none)
+//   acc = alpha_next x                         (where the next part adds; alpha_next 0: left alone)
+// x may be null too (nobody reads the float32 rows). acc may be src itself (every element is read by
+// the thread that writes it, after the row's sum is done); x and y are other rows than src.
+template <class TOut>
+__global__ void postnorm_kernel(const float* src, const float* __restrict__ w, float* __restrict__ x,
+                                TOut* __restrict__ y, float* acc, int H, float eps, float alpha_next) {
+    __shared__ float red[16];
+    const size_t row = (size_t)blockIdx.x * H;
+    float inv = 1.0f;
+    if (w) {
+        float ss = 0.f;
+        for (int i = threadIdx.x; i < H; i += blockDim.x) {
+            const float v = src[row + i];
+            ss = fmaf(v, v, ss);
+        }
+        ss = hb_block_sum(ss, red);
+        inv = 1.0f / sqrtf(ss / (float)H + eps);
+    }
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        const float v = w ? src[row + i] * inv * w[i] : src[row + i];
+        if (x) x[row + i] = v;
+        if (y) y[row + i] = hb_from_float<TOut>(v);
+        if (alpha_next != 0.f) acc[row + i] = alpha_next * v;
+    }
+}
+
+extern "C" int hb_postnorm(const float* src, const float* w, float* x, void* y, int y_dtype, float* acc, int R, int H,
+                           float eps, float alpha_next, hipStream_t stream) {
+    HB_REQUIRE(alpha_next == 0.f || acc != nullptr, "postnorm: no rows for alpha x");
+    HB_REQUIRE(R > 0 && H > 0, "postnorm: empty input (R=%d, H=%d)", R, H);
+    HB_REQUIRE(y_dtype == HB_F32 || y_dtype == HB_BF16, "postnorm: unknown output dtype %d", y_dtype);
+    const int threads = H >= 2048 ? 256 : H >= 512 ? 128 : 64;
+    if (y_dtype == HB_F32)
+        postnorm_kernel<float><<<R, threads, 0, stream>>>(src, w, x, (float*)y, acc, H, eps, alpha_next);
+    else
+        postnorm_kernel<bf16><<<R, threads, 0, stream>>>(src, w, x, (bf16*)y, acc, H, eps, alpha_next);
+    HB_CHECK_LAUNCH("postnorm");
+    return 0;
+}
+
+// ---------------------------------------------------------------- squared relu
+// act[i] = max(z[i], 0)^2, float32 in, any storage type out.
+template <class TOut>
+__global__ void relu_squared_kernel(const float* __restrict__ z, TOut* __restrict__ act, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        const float r = fmaxf(z[i], 0.f);
+        act[i] = hb_from_float<TOut>(r * r);
+    }
+}
+
+extern "C" int hb_relu_squared(const float* z, void* act, int act_dtype, size_t n, hipStream_t stream) {
+    HB_REQUIRE(n > 0, "relu_squared: empty input");
+    const size_t blocks = (n + 255) / 256;
+    const unsigned grid = (unsigned)(blocks > 16384 ? 16384 : blocks);
+    if (act_dtype == HB_F32)
+        relu_squared_kernel<float><<<grid, 256, 0, stream>>>(z, (float*)act, n);
+    else if (act_dtype == HB_BF16)
+        relu_squared_kernel<bf16><<<grid, 256, 0, stream>>>(z, (bf16*)act, n);
+    else
+        HB_REQUIRE(false, "relu_squared: unknown output dtype %d", act_dtype);
+    HB_CHECK_LAUNCH("relu_squared");
     return 0;
 }

@@ -5,7 +5,8 @@
 //             are consecutive, and a list of row tiles (expert, first row, rows) of fixed length
 //   products  a tile's rows times its expert's matrix, float32 sums over k ascending by one
 //             thread each (plain), whatever else is in the batch
-//   activate  g = min(gate, limit), u = clamp(up, -limit, limit): y = g sigmoid(alpha g) (u + 1)
+//   activate  g = min(gate, limit), u = clamp(up, -limit, limit): y = g sigmoid(alpha g) (u + shift)
+//             (limit infinite, alpha 1, shift 0: silu(gate) up)
 //   combine   a token's rows weighted and summed in the order of its choices, added to the output
 // Nothing here asks the host: the grids depend on the step's size only, so a step can be recorded
 // and replayed.
@@ -22,14 +23,14 @@ HB_MODULE_ERROR_SLOT()
 // ------------------------------------------------------------------------ route
 // One wave a token; lane l holds the logits of experts l, l + 64, ...
 __global__ void __launch_bounds__(HB_WAVE)
-moe_route_kernel(const float* __restrict__ logits, const float* __restrict__ bias, int* __restrict__ chosen,
+moe_route_kernel(const float* __restrict__ logits, int ld, const float* __restrict__ bias, int* __restrict__ chosen,
                  float* __restrict__ weight, int E, int top) {
     const int t = blockIdx.x, lane = threadIdx.x;
     float z[MOE_MAX_E_PER_LANE];
 #pragma unroll
     for (int i = 0; i < MOE_MAX_E_PER_LANE; ++i) {
         const int e = lane + HB_WAVE * i;
-        z[i] = e < E ? logits[(size_t)t * E + e] + (bias ? bias[e] : 0.f) : -INFINITY;
+        z[i] = e < E ? logits[(size_t)t * ld + e] + (bias ? bias[e] : 0.f) : -INFINITY;
     }
     float first = 0.f, sum = 0.f;
     for (int j = 0; j < top; ++j) {
@@ -64,6 +65,90 @@ moe_route_kernel(const float* __restrict__ logits, const float* __restrict__ bia
             if (lane + HB_WAVE * i == at) z[i] = -INFINITY;
     }
     for (int j = lane; j < top; j += HB_WAVE) weight[(size_t)t * top + j] /= sum;
+}
+
+// Routing by scores s = sigmoid(logit). The choice runs on s + correction, the weights on s itself:
+// the experts form n_groups equal groups of neighbours, a group is worth the sum of its two largest
+// choice scores, only the experts of the `keep` best groups can be chosen (the lower index of equals,
+// for groups as for experts), and the chosen experts' scores are divided by their sum + 1e-20.
+// One wave a token; the scores lie in LDS.
+__global__ void __launch_bounds__(HB_WAVE)
+moe_route_scores_kernel(const float* __restrict__ logits, int ld, const float* __restrict__ correction,
+                        int* __restrict__ chosen, float* __restrict__ weight, int E, int top, int n_groups,
+                        int keep) {
+    __shared__ float score[HB_WAVE * MOE_MAX_E_PER_LANE];
+    __shared__ float choice[HB_WAVE * MOE_MAX_E_PER_LANE];
+    __shared__ float worth[HB_WAVE * MOE_MAX_E_PER_LANE];
+    __shared__ int kept[HB_WAVE * MOE_MAX_E_PER_LANE];
+    const int t = blockIdx.x, lane = threadIdx.x;
+    const int size = E / n_groups;
+    for (int e = lane; e < E; e += HB_WAVE) {
+        const float s = 1.0f / (1.0f + expf(-logits[(size_t)t * ld + e]));
+        score[e] = s;
+        choice[e] = s + (correction ? correction[e] : 0.f);
+    }
+    __syncthreads();
+    for (int g = lane; g < n_groups; g += HB_WAVE) {
+        float a = -INFINITY, b = -INFINITY;          // the largest and the second
+        for (int i = 0; i < size; ++i) {
+            const float c = choice[g * size + i];
+            if (c > a) {
+                b = a;
+                a = c;
+            } else if (c > b) {
+                b = c;
+            }
+        }
+        worth[g] = size > 1 ? a + b : a;
+    }
+    __syncthreads();
+    for (int g = lane; g < n_groups; g += HB_WAVE) {
+        int ahead = 0;
+        for (int o = 0; o < n_groups; ++o) ahead += (worth[o] > worth[g] || (worth[o] == worth[g] && o < g)) ? 1 : 0;
+        kept[g] = ahead < keep;
+    }
+    __syncthreads();
+    float z[MOE_MAX_E_PER_LANE];
+#pragma unroll
+    for (int i = 0; i < MOE_MAX_E_PER_LANE; ++i) {
+        const int e = lane + HB_WAVE * i;
+        z[i] = (e < E && kept[e / size]) ? choice[e] : -INFINITY;
+    }
+    float sum = 0.f;
+    for (int j = 0; j < top; ++j) {
+        float best = -INFINITY;
+        int at = 0x7fffffff;
+#pragma unroll
+        for (int i = 0; i < MOE_MAX_E_PER_LANE; ++i) {
+            const int e = lane + HB_WAVE * i;
+            // (experts outside the kept groups and those already taken are never met: they are marked below)
+            if (e < E && z[i] != -INFINITY && (z[i] > best || at == 0x7fffffff || (z[i] == best && e < at))) {
+                best = z[i];
+                at = e;
+            }
+        }
+#pragma unroll
+        for (int off = HB_WAVE / 2; off > 0; off >>= 1) {
+            const float ob = __shfl_xor(best, off, HB_WAVE);
+            const int oa = __shfl_xor(at, off, HB_WAVE);
+            if (oa != 0x7fffffff && (at == 0x7fffffff || ob > best || (ob == best && oa < at))) {
+                best = ob;
+                at = oa;
+            }
+        }
+        if (at == 0x7fffffff) at = 0;                // (fewer experts in the kept groups than `top`: the host refuses that)
+        const float s = score[at];
+        sum += s;
+        if (lane == j % HB_WAVE) {
+            chosen[(size_t)t * top + j] = at;
+            weight[(size_t)t * top + j] = s;
+        }
+#pragma unroll
+        for (int i = 0; i < MOE_MAX_E_PER_LANE; ++i)
+            if (lane + HB_WAVE * i == at) z[i] = -INFINITY;
+    }
+    const float total = sum + 1e-20f;
+    for (int j = lane; j < top; j += HB_WAVE) weight[(size_t)t * top + j] /= total;
 }
 
 // ------------------------------------------------------------------------ group
@@ -122,15 +207,26 @@ moe_place_kernel(const int* __restrict__ chosen, int* __restrict__ counts, int* 
     }
 }
 
+// logits' rows are ld floats apart (their first E count).
+// by_scores 0: the largest logits (+ bias), weights a softmax over the chosen.
+// by_scores 1: sigmoid scores, `bias` is the correction of the choice, n_groups groups of which `keep` count.
 extern "C" int hb_moe_route(const float* logits, const float* bias, int* chosen, float* weight, int* counts,
                             int* order, int* row_of, int* tile_expert, int* tile_row0, int* tile_rows, int T, int E,
-                            int top, int max_tiles, hipStream_t stream) {
+                            int top, int max_tiles, int ld, int by_scores, int n_groups, int keep,
+                            hipStream_t stream) {
+    HB_REQUIRE(ld >= E, "moe: logits rows %d apart for %d experts", ld, E);
+    HB_REQUIRE(!by_scores || (n_groups > 0 && E % n_groups == 0 && keep > 0 && keep <= n_groups &&
+                              top <= keep * (E / n_groups)),
+               "moe: %d of %d groups of %d experts cannot give %d experts", keep, n_groups, E, top);
     HB_REQUIRE(T > 0 && E > 0 && top > 0 && top <= E, "moe: %d of %d experts for %d tokens", top, E, T);
     HB_REQUIRE(E <= HB_WAVE * MOE_MAX_E_PER_LANE, "moe: %d experts, the router takes up to %d", E, HB_WAVE * MOE_MAX_E_PER_LANE);
     const long long A = (long long)T * top;
     HB_REQUIRE(A < (1ll << 30), "moe: too many (token, expert) pairs");
     HB_REQUIRE(max_tiles >= (A + MOE_TILE_M - 1) / MOE_TILE_M + E, "moe: the tile list is too short");
-    moe_route_kernel<<<T, HB_WAVE, 0, stream>>>(logits, bias, chosen, weight, E, top);
+    if (by_scores)
+        moe_route_scores_kernel<<<T, HB_WAVE, 0, stream>>>(logits, ld, bias, chosen, weight, E, top, n_groups, keep);
+    else
+        moe_route_kernel<<<T, HB_WAVE, 0, stream>>>(logits, ld, bias, chosen, weight, E, top);
     HB_CHECK_LAUNCH("moe_route");
     moe_place_kernel<<<E + 1, 256, 0, stream>>>(chosen, counts, order, row_of, tile_expert, tile_row0, tile_rows, (int)A, E, max_tiles);
     HB_CHECK_LAUNCH("moe_place");
@@ -227,26 +323,26 @@ extern "C" int hb_moe_gemm_plain(const void* A, int a_dtype, const void* W, int 
 // gu [pairs, 2 F] float32 (gate columns, then up columns) -> act [pairs, F]
 template <class TOut>
 __global__ void moe_activate_kernel(const float* __restrict__ gu, TOut* __restrict__ act, int F, size_t total,
-                                    float limit, float alpha) {
+                                    float limit, float alpha, float shift) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
         const size_t r = i / F;
         const int n = (int)(i % F);
         const float g = fminf(gu[r * 2 * F + n], limit);
         const float u = fminf(fmaxf(gu[r * 2 * F + F + n], -limit), limit);
-        act[i] = hb_from_float<TOut>(g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+        act[i] = hb_from_float<TOut>(g / (1.0f + expf(-alpha * g)) * (u + shift));
     }
 }
 
 extern "C" int hb_moe_activate(const float* gu, void* act, int act_dtype, int rows, int F, float limit, float alpha,
-                               hipStream_t stream) {
+                               float shift, hipStream_t stream) {
     HB_REQUIRE(rows > 0 && F > 0, "moe activation: empty input");
     const size_t total = (size_t)rows * F;
     const size_t blocks = (total + 255) / 256;
     const unsigned grid = (unsigned)(blocks > 8192 ? 8192 : blocks);
     if (act_dtype == HB_F32)
-        moe_activate_kernel<float><<<grid, 256, 0, stream>>>(gu, (float*)act, F, total, limit, alpha);
+        moe_activate_kernel<float><<<grid, 256, 0, stream>>>(gu, (float*)act, F, total, limit, alpha, shift);
     else if (act_dtype == HB_BF16)
-        moe_activate_kernel<bf16><<<grid, 256, 0, stream>>>(gu, (bf16*)act, F, total, limit, alpha);
+        moe_activate_kernel<bf16><<<grid, 256, 0, stream>>>(gu, (bf16*)act, F, total, limit, alpha, shift);
     else
         HB_REQUIRE(false, "moe activation: unknown output dtype %d", act_dtype);
     HB_CHECK_LAUNCH("moe_activate");
@@ -255,9 +351,12 @@ extern "C" int hb_moe_activate(const float* gu, void* act, int act_dtype, int ro
 
 // ------------------------------------------------------------------------ combine
 // x[t, :] += sum_j weight[t, j] * y[row_of[t * top + j], :]    (float32, j ascending)
+// shared [T, H] (or null): a part that every token takes, added times sigmoid(gate[t * gate_ld]).
 __global__ void moe_combine_kernel(const float* __restrict__ y, const float* __restrict__ weight,
-                                   const int* __restrict__ row_of, float* __restrict__ x, int top, int H) {
+                                   const int* __restrict__ row_of, float* __restrict__ x, int top, int H,
+                                   const float* __restrict__ shared, const float* __restrict__ gate, int gate_ld) {
     const int t = blockIdx.x;
+    const float open = shared ? 1.0f / (1.0f + expf(-gate[(size_t)t * gate_ld])) : 0.f;
     // (a token's rows and weights once, eight at a time, then whole rows)
     for (int j0 = 0; j0 < top; j0 += 8) {
         const float* rows[8];
@@ -273,15 +372,17 @@ __global__ void moe_combine_kernel(const float* __restrict__ y, const float* __r
 #pragma unroll
             for (int j = 0; j < 8; ++j)
                 if (j0 + j < top) s = fmaf(w[j], rows[j][i], s);
+            if (shared && j0 == 0) s = fmaf(open, shared[(size_t)t * H + i], s);
             x[(size_t)t * H + i] += s;
         }
     }
 }
 
 extern "C" int hb_moe_combine(const float* y, const float* weight, const int* row_of, float* x, int T, int top, int H,
-                              hipStream_t stream) {
+                              const float* shared, const float* gate, int gate_ld, hipStream_t stream) {
+    HB_REQUIRE(shared == nullptr || (gate != nullptr && gate_ld > 0), "moe combine: a shared part needs its gate");
     HB_REQUIRE(T > 0 && top > 0 && H > 0, "moe combine: empty input");
-    moe_combine_kernel<<<T, H >= 1024 ? 256 : 64, 0, stream>>>(y, weight, row_of, x, top, H);
+    moe_combine_kernel<<<T, H >= 1024 ? 256 : 64, 0, stream>>>(y, weight, row_of, x, top, H, shared, gate, gate_ld);
     HB_CHECK_LAUNCH("moe_combine");
     return 0;
 }
@@ -304,7 +405,7 @@ extern "C" int hb_moe_combine(const float* y, const float* weight, const int* ro
 // An output is summed over k in the same order whatever else the tile holds.
 // EPI 0: float32 C. EPI 1: bfloat16 C. EPI 2: W[g] is [2 F, K], gate rows then up rows; a wave's two
 // blocks are 16 gate rows and the 16 up rows that go with them, and C [*, F] bfloat16 receives
-// min(gate, limit) sigmoid(alpha min(gate, limit)) (clamp(up, -limit, limit) + 1).
+// min(gate, limit) sigmoid(alpha min(gate, limit)) (clamp(up, -limit, limit) + shift).
 typedef __bf16 hb_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float hb_f32x4 __attribute__((ext_vector_type(4)));
 
@@ -315,7 +416,7 @@ __global__ void __launch_bounds__(256)
 grouped_mfma_kernel(const bf16* __restrict__ A, int lda, size_t a_group_off, const bf16* __restrict__ W, int N,
                     int K, void* __restrict__ Cv, int ldc, size_t c_group_off, const int* __restrict__ order,
                     int top, const int* __restrict__ tile_group, const int* __restrict__ tile_row0,
-                    const int* __restrict__ tile_rows, int M, int m_tiles, float limit, float alpha) {
+                    const int* __restrict__ tile_rows, int M, int m_tiles, float limit, float alpha, float shift) {
     // the tile's activations, a stage of 64 k at a time, as 16-byte pieces [k piece][row]: a wave's operand
     // (16 rows of one piece) is 256 contiguous bytes
     __shared__ __attribute__((aligned(16))) hb_bf16x8 a_lds[2][GM_KSTEP / 8][MOE_TILE_M];
@@ -421,7 +522,7 @@ grouped_mfma_kernel(const bf16* __restrict__ A, int lda, size_t a_group_off, con
                     if (n >= F) continue;
                     const float g = fminf(acc[a][b][i], limit);
                     const float u = fminf(fmaxf(acc[a + 2][b][i], -limit), limit);
-                    C[base + n] = hb_from_float<bf16>(g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+                    C[base + n] = hb_from_float<bf16>(g / (1.0f + expf(-alpha * g)) * (u + shift));
                 }
         } else {
 #pragma unroll
@@ -446,7 +547,7 @@ __global__ void __launch_bounds__(256)
 grouped_mfma_stream_kernel(const bf16* __restrict__ A, int lda, size_t a_group_off, const bf16* __restrict__ W, int N,
                     int K, void* __restrict__ Cv, int ldc, size_t c_group_off, const int* __restrict__ order,
                     int top, const int* __restrict__ tile_group, const int* __restrict__ tile_row0,
-                    const int* __restrict__ tile_rows, int M, int m_tiles, float limit, float alpha) {
+                    const int* __restrict__ tile_rows, int M, int m_tiles, float limit, float alpha, float shift) {
     int group, row0, rows;
     if (tile_group) {
         group = tile_group[blockIdx.y];
@@ -519,7 +620,7 @@ grouped_mfma_stream_kernel(const bf16* __restrict__ A, int lda, size_t a_group_o
                 if (n >= F) continue;
                 const float g = fminf(acc[0][b][i], limit);
                 const float u = fminf(fmaxf(acc[1][b][i], -limit), limit);
-                C[base + n] = hb_from_float<bf16>(g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+                C[base + n] = hb_from_float<bf16>(g / (1.0f + expf(-alpha * g)) * (u + shift));
             }
         } else {
 #pragma unroll
@@ -543,7 +644,7 @@ grouped_mfma_stream_kernel(const bf16* __restrict__ A, int lda, size_t a_group_o
 extern "C" int hb_grouped_mfma(const void* A, int lda, size_t a_group_off, const void* W, int N, int K, void* C,
                                int ldc, size_t c_group_off, int epi, const int* order, int top,
                                const int* tile_group, const int* tile_row0, const int* tile_rows, int n_tiles, int M,
-                               int groups, float limit, float alpha, int few_rows, hipStream_t stream) {
+                               int groups, float limit, float alpha, float shift, int few_rows, hipStream_t stream) {
     HB_REQUIRE(N > 0 && K > 0 && K % 32 == 0, "grouped product: K = %d must be a positive multiple of 32", K);
     HB_REQUIRE(N % 16 == 0 && (epi != 2 || N % 32 == 0), "grouped product: %d weight rows are no whole blocks of 16", N);
     HB_REQUIRE(lda % 8 == 0 && a_group_off % 8 == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0,
@@ -563,7 +664,7 @@ extern "C" int hb_grouped_mfma(const void* A, int lda, size_t a_group_off, const
 #define HB_GROUPED_STREAM(E)                                                                                        \
     grouped_mfma_stream_kernel<E><<<grid, 256, 0, stream>>>((const bf16*)A, lda, a_group_off, (const bf16*)W, N, K, \
                                                             C, ldc, c_group_off, order, top, tile_group, tile_row0,  \
-                                                            tile_rows, M, m_tiles, limit, alpha)
+                                                            tile_rows, M, m_tiles, limit, alpha, shift)
     if (few_rows) {
         if (epi == 0) HB_GROUPED_STREAM(0);
         else if (epi == 1) HB_GROUPED_STREAM(1);
@@ -575,7 +676,7 @@ extern "C" int hb_grouped_mfma(const void* A, int lda, size_t a_group_off, const
 #define HB_GROUPED(E)                                                                                               \
     grouped_mfma_kernel<E><<<grid, 256, 0, stream>>>((const bf16*)A, lda, a_group_off, (const bf16*)W, N, K, C, ldc, \
                                                      c_group_off, order, top, tile_group, tile_row0, tile_rows, M,   \
-                                                     m_tiles, limit, alpha)
+                                                     m_tiles, limit, alpha, shift)
     if (epi == 0) HB_GROUPED(0);
     else if (epi == 1) HB_GROUPED(1);
     else HB_GROUPED(2);

@@ -112,8 +112,10 @@ extern "C" int hb_conv_silu(const float* proj, int ld, const float* taps, float*
 // Tokens that are loaded together, and such groups in the ring. A group's loads are issued before the
 // group that is worked on and waited for after it, so a group must take longer than the memory's latency:
 // with 8 tokens a group the kernel took that latency over 8 a token. (8 where 16 would not fit 64 KB of LDS.)
-#define DELTA_SUB_OF(DP) ((DP) >= 256 ? 8 : 16)
-#define DELTA_RING_OF(LPC) 3
+// CH: the decay is a factor a row of S (a key channel) instead of one a head: decay [T, heads x D] holds
+// the factors themselves (hb_channel_decay makes them), and they come through the ring beside k and q.
+#define DELTA_SUB_OF(DP, CH) ((CH) ? ((DP) >= 128 ? 8 : 16) : ((DP) >= 256 ? 8 : 16))
+#define DELTA_RING_OF(DP, CH) (((CH) && (DP) >= 256) ? 2 : 3)
 
 __device__ __forceinline__ float delta_dpp(float v, const int ctrl) {
     // (a lane reads another lane's value: ctrl names which, within rows of 16 lanes)
@@ -136,21 +138,24 @@ __device__ __forceinline__ float delta_column_sum(float v) {
     return v;
 }
 
-template <int LPC, int DELTA_PER>
+template <int LPC, int DELTA_PER, bool CH>
 __global__ void __launch_bounds__(HB_WAVE)
 gated_delta_kernel(const float* __restrict__ qkv, int C, const float* __restrict__ proj, int ld, int b_off,
                    int a_off, const float* __restrict__ A_log, const float* __restrict__ dt_bias,
-                   float* __restrict__ state, const int* __restrict__ seq_starts, const int* __restrict__ slots,
+                   const float* __restrict__ decay, float* __restrict__ state,
+                   const int* __restrict__ seq_starts, const int* __restrict__ slots,
                    float* __restrict__ out, int kv_heads, int heads, int D, int V) {
     constexpr int COLS = HB_WAVE / LPC;
     constexpr int DP = LPC * DELTA_PER;                 // D rounded up to what the lanes hold
-    constexpr int DELTA_RING = DELTA_RING_OF(LPC);
-    constexpr int DELTA_SUB = DELTA_SUB_OF(LPC * DELTA_PER);
+    constexpr int DELTA_RING = DELTA_RING_OF(DP, CH);
+    constexpr int DELTA_SUB = DELTA_SUB_OF(DP, CH);
     constexpr int SLOTS = DELTA_SUB * DELTA_RING;
-    constexpr int KQ4 = DELTA_SUB * DP / 2;             // float4 of k and q a group of tokens
+    constexpr int NB = CH ? 3 : 2;                      // blocks of DP numbers a token in the ring: k, q (, decay)
+    constexpr int ROW4 = NB * DP / 4;                   // float4 of a token's ring row
+    constexpr int KQ4 = DELTA_SUB * ROW4;               // float4 of k and q (and the decays) a group of tokens
     constexpr int KQ_PER_LANE = (KQ4 + HB_WAVE - 1) / HB_WAVE;
     constexpr int V_PER_LANE = (DELTA_SUB * COLS + HB_WAVE - 1) / HB_WAVE;
-    __shared__ __attribute__((aligned(16))) float kq_ring[SLOTS][2 * DP];
+    __shared__ __attribute__((aligned(16))) float kq_ring[SLOTS][NB * DP];
     __shared__ float v_ring[SLOTS][COLS];
     __shared__ float gb_ring[SLOTS][2];
     const int seq = blockIdx.x, h = blockIdx.y;
@@ -169,8 +174,9 @@ gated_delta_kernel(const float* __restrict__ qkv, int C, const float* __restrict
     // (numbers beyond D are zeros and stay zeros: their k and q are zeros in the ring)
 #pragma unroll
     for (int i = 0; i < DELTA_PER; ++i) S[i] = (live && d0 + i < D) ? S_mem[(size_t)(d0 + i) * V] : 0.f;
-    const float rate = -expf(A_log[h]);
-    const float bias = dt_bias[h];
+    const float rate = CH ? 0.f : -expf(A_log[h]);
+    const float bias = CH ? 0.f : dt_bias[h];
+    const int g_ld = heads * D;
     const int q_at = kvh * D, k_at = (kv_heads + kvh) * D, v_at = 2 * kv_heads * D + h * V;
     const bool vec = (D % 4) == 0 && (C % 4) == 0;
 
@@ -182,11 +188,13 @@ gated_delta_kernel(const float* __restrict__ qkv, int C, const float* __restrict
 #pragma unroll
         for (int j = 0; j < KQ_PER_LANE; ++j) {
             const int idx = j * HB_WAVE + lane;
-            const int i = idx / (DP / 2), f = idx % (DP / 2);        // token of the group, float4 of its [k | q]
+            const int i = idx / ROW4, f = idx % ROW4;               // token of the group, float4 of its [k | q (| decay)]
             const int d = 4 * (f % (DP / 4));
+            const int block = f / (DP / 4);
             float4 r = float4{0.f, 0.f, 0.f, 0.f};
             if (idx < KQ4 && t0 + i < last) {
-                const float* src = qkv + (size_t)(t0 + i) * C + (f < DP / 4 ? k_at : q_at) + d;
+                const float* src = (CH && block == 2) ? decay + (size_t)(t0 + i) * g_ld + (size_t)h * D + d
+                                                      : qkv + (size_t)(t0 + i) * C + (block == 0 ? k_at : q_at) + d;
                 if (vec && d + 3 < D) {
                     r = *(const float4*)src;
                 } else {
@@ -206,9 +214,11 @@ gated_delta_kernel(const float* __restrict__ qkv, int C, const float* __restrict
                             ? qkv[(size_t)(t0 + i) * C + v_at + col0 + c] : 0.f;
         }
         if (lane < DELTA_SUB && t0 + lane < last) {
-            const float z = proj[(size_t)(t0 + lane) * ld + a_off + h] + bias;
-            const float softplus = z > 20.f ? z : log1pf(expf(z));
-            g_reg = expf(rate * softplus);
+            if (!CH) {
+                const float z = proj[(size_t)(t0 + lane) * ld + a_off + h] + bias;
+                const float softplus = z > 20.f ? z : log1pf(expf(z));
+                g_reg = expf(rate * softplus);
+            }
             beta_reg = 1.0f / (1.0f + expf(-proj[(size_t)(t0 + lane) * ld + b_off + h]));
         }
     };
@@ -218,7 +228,7 @@ gated_delta_kernel(const float* __restrict__ qkv, int C, const float* __restrict
 #pragma unroll
         for (int j = 0; j < KQ_PER_LANE; ++j) {
             const int idx = j * HB_WAVE + lane;
-            if (idx < KQ4) *(float4*)&kq_ring[s0 + idx / (DP / 2)][4 * (idx % (DP / 2))] = kq_regs[j];
+            if (idx < KQ4) *(float4*)&kq_ring[s0 + idx / ROW4][4 * (idx % ROW4)] = kq_regs[j];
         }
 #pragma unroll
         for (int j = 0; j < V_PER_LANE; ++j) {
@@ -252,6 +262,28 @@ gated_delta_kernel(const float* __restrict__ qkv, int C, const float* __restrict
             }
             const float vc = v_ring[s0 + i][lcol];
             const float g = gb_ring[s0 + i][0], beta = gb_ring[s0 + i][1];
+            if (CH) {
+                // a factor a row: the numbers decay first, then both dot products run on them
+                float d4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int e = 0; e < DELTA_PER; e += 4) {
+                    const float4 gg = *(const float4*)&kq_ring[s0 + i][2 * DP + d0 + e];
+                    S[e] *= gg.x, S[e + 1] *= gg.y, S[e + 2] *= gg.z, S[e + 3] *= gg.w;
+                }
+#pragma unroll
+                for (int e = 0; e < DELTA_PER; ++e) d4[e & 3] = fmaf(S[e], kc[e], d4[e & 3]);
+                const float dot = delta_column_sum<LPC>((d4[0] + d4[1]) + (d4[2] + d4[3]));
+                const float u = beta * (vc - dot);
+                float o4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int e = 0; e < DELTA_PER; ++e) {
+                    S[e] = fmaf(kc[e], u, S[e]);
+                    o4[e & 3] = fmaf(S[e], qc[e], o4[e & 3]);
+                }
+                const float o = delta_column_sum<LPC>((o4[0] + o4[1]) + (o4[2] + o4[3]));
+                if (live && part == 0) out[(size_t)(t0 + i) * heads * V + h * V + col] = o;
+                continue;
+            }
             // g (S^T k) = (g S)^T k: the dot product runs on the old numbers, in four partial sums, and the
             // decay of the numbers themselves does not wait for it
             float d4[4] = {0.f, 0.f, 0.f, 0.f};
@@ -278,8 +310,11 @@ gated_delta_kernel(const float* __restrict__ qkv, int C, const float* __restrict
     }
 }
 
+// decay null: one factor a head, from the projection's column a_off + h, A_log and dt_bias.
+// decay [T, heads x D]: a factor a key channel, as given (a_off, A_log and dt_bias are not read).
 extern "C" int hb_gated_delta(const float* qkv, int C, const float* proj, int ld, int b_off, int a_off,
-                              const float* A_log, const float* dt_bias, float* state, const int* seq_starts,
+                              const float* A_log, const float* dt_bias, const float* decay, float* state,
+                              const int* seq_starts,
                               const int* slots, float* out, int B, int kv_heads, int heads, int D, int V,
                               hipStream_t stream) {
     HB_REQUIRE(B > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "delta rule: %d heads on %d key heads", heads, kv_heads);
@@ -297,8 +332,14 @@ extern "C" int hb_gated_delta(const float* qkv, int C, const float* proj, int ld
     const int cols = HB_WAVE / lpc;
     const dim3 grid(B, heads, (V + cols - 1) / cols);
 #define HB_DELTA(L, P)                                                                                            \
-    gated_delta_kernel<L, P><<<grid, HB_WAVE, 0, stream>>>(qkv, C, proj, ld, b_off, a_off, A_log, dt_bias, state,  \
-                                                           seq_starts, slots, out, kv_heads, heads, D, V)
+    do {                                                                                                          \
+        if (decay)                                                                                                \
+            gated_delta_kernel<L, P, true><<<grid, HB_WAVE, 0, stream>>>(qkv, C, proj, ld, b_off, a_off, A_log,   \
+                dt_bias, decay, state, seq_starts, slots, out, kv_heads, heads, D, V);                            \
+        else                                                                                                      \
+            gated_delta_kernel<L, P, false><<<grid, HB_WAVE, 0, stream>>>(qkv, C, proj, ld, b_off, a_off, A_log,  \
+                dt_bias, decay, state, seq_starts, slots, out, kv_heads, heads, D, V);                            \
+    } while (0)
     if (wide) {
         if (lpc == 1) HB_DELTA(1, 8);
         else if (lpc == 2) HB_DELTA(2, 8);
@@ -318,12 +359,13 @@ extern "C" int hb_gated_delta(const float* qkv, int C, const float* proj, int ld
 }
 
 // ------------------------------------- norm a head, weight, gate: what leaves the recurrence
-// y[t, h, :] = o / sqrt(mean(o^2) + eps) * w * silu(gate[t, h, :]); w [V] is shared by the heads,
+// y[t, h, :] = o / sqrt(mean(o^2) + eps) * w * silu(gate[t, h, :]) (or sigmoid(gate), if so asked); w [V] is shared by the heads,
 // the gate's pre-activations are columns [g_off + h V, ...) of the projection's row. One wave a (token, head).
 template <class TOut>
 __global__ void __launch_bounds__(HB_WAVE)
 gated_head_norm_kernel(const float* __restrict__ o, const float* __restrict__ proj, int ld, int g_off,
-                       const float* __restrict__ w, TOut* __restrict__ y, int heads, int V, float eps) {
+                       const float* __restrict__ w, TOut* __restrict__ y, int heads, int V, float eps,
+                       int sigmoid_gate) {
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const float* in = o + ((size_t)t * heads + h) * V;
     const float* gate = proj + (size_t)t * ld + g_off + (size_t)h * V;
@@ -332,18 +374,48 @@ gated_head_norm_kernel(const float* __restrict__ o, const float* __restrict__ pr
     for (int d = lane; d < V; d += HB_WAVE) ss = fmaf(in[d], in[d], ss);
     ss = hb_wave_sum(ss);
     const float inv = 1.0f / sqrtf(ss / (float)V + eps);
-    for (int d = lane; d < V; d += HB_WAVE) out[d] = hb_from_float<TOut>(in[d] * inv * w[d] * hb_silu(gate[d]));
+    for (int d = lane; d < V; d += HB_WAVE) {
+        const float z = gate[d];
+        const float open = sigmoid_gate ? 1.0f / (1.0f + expf(-z)) : hb_silu(z);
+        out[d] = hb_from_float<TOut>(in[d] * inv * w[d] * open);
+    }
 }
 
 extern "C" int hb_gated_head_norm(const float* o, const float* proj, int ld, int g_off, const float* w, void* y,
-                                  int y_dtype, int T, int heads, int V, float eps, hipStream_t stream) {
+                                  int y_dtype, int T, int heads, int V, float eps, int sigmoid_gate,
+                                  hipStream_t stream) {
     HB_REQUIRE(T > 0 && heads > 0 && V > 0 && heads <= 65535, "gated norm: empty input or too many heads");
     if (y_dtype == HB_F32)
-        gated_head_norm_kernel<float><<<dim3(T, heads), HB_WAVE, 0, stream>>>(o, proj, ld, g_off, w, (float*)y, heads, V, eps);
+        gated_head_norm_kernel<float><<<dim3(T, heads), HB_WAVE, 0, stream>>>(o, proj, ld, g_off, w, (float*)y, heads, V, eps, sigmoid_gate);
     else if (y_dtype == HB_BF16)
-        gated_head_norm_kernel<bf16><<<dim3(T, heads), HB_WAVE, 0, stream>>>(o, proj, ld, g_off, w, (bf16*)y, heads, V, eps);
+        gated_head_norm_kernel<bf16><<<dim3(T, heads), HB_WAVE, 0, stream>>>(o, proj, ld, g_off, w, (bf16*)y, heads, V, eps, sigmoid_gate);
     else
         HB_REQUIRE(false, "gated norm: unknown output dtype %d", y_dtype);
     HB_CHECK_LAUNCH("gated_head_norm");
+    return 0;
+}
+
+// ------------------------------------------------- a decay a key channel from its pre-activation
+// g[t, h, d] = exp(-exp(A_log[h]) * softplus(z[t, h, d] + dt_bias[h, d])), float32; z's rows are ld apart
+// (g's are heads x D apart, and g may be z itself where ld is that).
+__global__ void channel_decay_kernel(const float* z, int ld, const float* __restrict__ A_log,
+                                     const float* __restrict__ dt_bias, float* g, int D, int HD, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t t = i / HD;
+        const int c = (int)(i - t * HD);
+        const float a = z[t * ld + c] + dt_bias[c];
+        const float softplus = a > 20.f ? a : log1pf(expf(a));
+        g[i] = expf(-expf(A_log[c / D]) * softplus);
+    }
+}
+
+extern "C" int hb_channel_decay(const float* z, int ld, const float* A_log, const float* dt_bias, float* g, int T,
+                                int heads, int D, hipStream_t stream) {
+    HB_REQUIRE(T > 0 && heads > 0 && D > 0 && ld >= heads * D, "channel decay: empty input");
+    const size_t n = (size_t)T * heads * D;
+    const size_t blocks = (n + 255) / 256;
+    channel_decay_kernel<<<(unsigned)(blocks > 16384 ? 16384 : blocks), 256, 0, stream>>>(z, ld, A_log, dt_bias, g,
+                                                                                           D, heads * D, n);
+    HB_CHECK_LAUNCH("channel_decay");
     return 0;
 }

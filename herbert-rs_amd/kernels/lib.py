@@ -23,11 +23,13 @@ SIGNATURES = {
         "hb_embed": [_P, _P, _I, _P, _I, _I, _I, _I, _P],
         "hb_rmsnorm": [_P, _P, _P, _I, _P, _I, _I, _F, _P],
         "hb_qk_norm_rope_write": [_P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _P, _P, _P, _I,
-                                  _I, _I, _I, _I, _F, _I, _I, ctypes.c_size_t, _P],
+                                  _I, _I, _I, _I, _F, _I, _I, ctypes.c_size_t, _F, _I, _P],
         "hb_swiglu": [_P, _P, _I, _I, _I, _P],
         "hb_fill_u32": [_P, _U32, _SZ, _P],
         "hb_layernorm": [_P, _P, _F, _P, _P, _I, _P, _I, _I, _F, _P],
         "hb_scale": [_P, _F, _SZ, _P],
+        "hb_postnorm": [_P, _P, _P, _P, _I, _P, _I, _I, _F, _F, _P],
+        "hb_relu_squared": [_P, _P, _I, _SZ, _P],
     },
     "gemm_plain": {
         "hb_gemm_plain": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P],
@@ -35,8 +37,9 @@ SIGNATURES = {
     },
     "recurrent": {
         "hb_conv_silu": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I, _I, _P],
-        "hb_gated_delta": [_P, _I, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
-        "hb_gated_head_norm": [_P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _P],
+        "hb_gated_delta": [_P, _I, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
+        "hb_gated_head_norm": [_P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _I, _P],
+        "hb_channel_decay": [_P, _I, _P, _P, _P, _I, _I, _I, _P],
     },
     "attention_latent": {
         "hb_latent_write": [_P, _I, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
@@ -44,11 +47,11 @@ SIGNATURES = {
         "hb_latent_attention_plain": [_P, _P, _P, _I, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P],
     },
     "moe": {
-        "hb_moe_route": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
+        "hb_moe_route": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P],
         "hb_moe_gemm_plain": [_P, _I, _P, _I, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _P],
-        "hb_moe_activate": [_P, _P, _I, _I, _I, _F, _F, _P],
-        "hb_moe_combine": [_P, _P, _P, _P, _I, _I, _I, _P],
-        "hb_grouped_mfma": [_P, _I, _SZ, _P, _I, _I, _P, _I, _SZ, _I, _P, _I, _P, _P, _P, _I, _I, _I, _F, _F, _I, _P],
+        "hb_moe_activate": [_P, _P, _I, _I, _I, _F, _F, _F, _P],
+        "hb_moe_combine": [_P, _P, _P, _P, _I, _I, _I, _P, _P, _I, _P],
+        "hb_grouped_mfma": [_P, _I, _SZ, _P, _I, _I, _P, _I, _SZ, _I, _P, _I, _P, _P, _P, _I, _I, _I, _F, _F, _F, _I, _P],
     },
     "attention_plain": {
         "hb_attention_plain": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],

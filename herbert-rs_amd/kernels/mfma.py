@@ -11,6 +11,7 @@ import torch
 
 from ..errors import BackendError
 from . import lib
+from . import ops
 from .ops import _check, _stream
 
 _P = ctypes.c_void_p
@@ -388,7 +389,7 @@ def gemm_swiglu(a, w_interleaved, out, packed=False, norm=None, tile=0, row_scal
 lib.register_signatures("attention_mfma", {
     "hb_attn_prefill_mfma": [_P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P],
     "hb_attn_decode_mfma": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I,
-                            _P, _P, _P, _P, _P, _F, _I, _I, ctypes.c_size_t, _P, _P],
+                            _P, _P, _P, _P, _P, _F, _I, _I, ctypes.c_size_t, _P, _F, _I, _P],
 })
 
 ATTENTION_HEAD_DIMS = (32, 64, 128)
@@ -535,14 +536,16 @@ def decode_fusable(meta, kv, nq, nkv, hd, rot_dims, dtype):
 
 
 def attention_decode_fused(qkv, q_norm_w, k_norm_w, cos, sin, meta, kv, out, nq, nkv, hd, eps, scale, window,
-                           qkv_slices=None, scratch=None):
+                           qkv_slices=None, scratch=None, q_temp=None):
     """One token a sequence: per-head norm (if weights are given), rotation (if tables are given),
     the new key and value written to the pages, and attention over them, in one kernel (+ merge).
     qkv f32 [B, (nq + 2 nkv) hd]; cos / sin f32 [max_pos, hd / 2]; out bf16 [B, nq hd].
     qkv_slices = (slices, pointer, floats between two), as gemm(..., defer_slices=True) returns it:
     the projection's sums are still in that many slices, which the kernel adds up as it loads them
-    (qkv itself is then not read)."""
+    (qkv itself is then not read). q_temp = (coef, every): a query at position p is multiplied by
+    1 + coef ln(floor((p + 1) / every) + 1) after its norm."""
     B = meta.num_seqs
+    coef, every = ops.query_temperature_args(q_temp)
     _check(qkv, "qkv", torch.float32, (B, (nq + 2 * nkv) * hd))
     _check(out, "out", torch.bfloat16, (B, nq * hd))
     pages = kv.k.shape[0]
@@ -580,7 +583,7 @@ def attention_decode_fused(qkv, q_norm_w, k_norm_w, cos, sin, meta, kv, out, nq,
              window, splits, per, src, None if q_norm_w is None else q_norm_w.data_ptr(),
              None if k_norm_w is None else k_norm_w.data_ptr(), None if cos is None else cos.data_ptr(),
              None if sin is None else sin.data_ptr(), float(eps), 1, n_slices, stride,
-             None if ranges is None else ranges.data_ptr(), _stream())
+             None if ranges is None else ranges.data_ptr(), coef, every, _stream())
 
 
 DEFERRED_SLICES = (2, 4, 8)     # numbers of slices of the projection that the decode kernel adds up itself
@@ -616,7 +619,7 @@ def attention(q, meta, kv, out, nq, nkv, hd, scale, window, tile_height=None, sc
                  out.data_ptr(), po.data_ptr(), pml.data_ptr(), meta.context_lens.data_ptr(),
                  meta.slots.data_ptr(), kv.page_table.data_ptr(), kv.page_table.shape[1], kv.page_size,
                  T, nq, nkv, hd, float(scale), window, splits, per, None, None, None, None, None, 0.0, 0, 1, 0,
-                 None if ranges is None else ranges.data_ptr(), _stream())
+                 None if ranges is None else ranges.data_ptr(), 0.0, 0, _stream())
         return
     _check(meta.positions, "positions", torch.int32, (T,))
     height = tile_height or _prefill_tile_height(meta, nkv, nq // nkv)

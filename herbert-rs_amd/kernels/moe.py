@@ -40,10 +40,20 @@ class Routing:
         return 3 * T * top + E + 3 * max_tiles(T * top, E)
 
 
-def route(logits, bias, routing):
-    """logits f32 [T, E] (+ bias f32 [E]) -> routing (see Routing)."""
+def route(logits, bias, routing, scores=False, groups=1, keep=1):
+    """logits f32 [T, E] (+ bias f32 [E]) -> routing (see Routing): the largest logits + bias, weighed by a
+    softmax over the chosen. The logits' rows may be wider than E (their first E columns count).
+    scores=True: s = sigmoid(logit), the choice runs on s + bias within the `keep` best of `groups` equal
+    groups of neighbours (a group is worth its two largest choice scores), and the weights are the chosen
+    experts' s over their sum."""
     r = routing
-    _check(logits, "logits", torch.float32, (r.T, r.E))
+    _check(logits, "logits", torch.float32, (r.T, None))
+    ld = logits.shape[1]
+    if ld < r.E:
+        raise BackendError(f"routing: logits of {ld} columns for {r.E} experts")
+    if scores and (groups <= 0 or r.E % groups or not 0 < keep <= groups
+                   or r.top > keep * (r.E // groups)):
+        raise BackendError(f"routing: {r.top} experts out of {keep} of {groups} groups of {r.E} experts")
     if bias is not None:
         _check(bias, "bias", torch.float32, (r.E,))
     _check(r.weight, "weight", torch.float32, (r.T, r.top))
@@ -51,7 +61,8 @@ def route(logits, bias, routing):
         raise BackendError(f"routing: {r.top} of {r.E} experts")
     lib.call("moe", "hb_moe_route", logits.data_ptr(), _ptr(bias), r.chosen.data_ptr(), r.weight.data_ptr(),
              r.counts.data_ptr(), r.order.data_ptr(), r.row_of.data_ptr(), r.tile_expert.data_ptr(),
-             r.tile_row0.data_ptr(), r.tile_rows.data_ptr(), r.T, r.E, r.top, r.tiles, _stream())
+             r.tile_row0.data_ptr(), r.tile_rows.data_ptr(), r.T, r.E, r.top, r.tiles, ld, 1 if scores else 0,
+             int(groups), int(keep), _stream())
 
 
 def gemm_plain(a, w, c, routing, gather):
@@ -67,26 +78,37 @@ def gemm_plain(a, w, c, routing, gather):
              r.tile_rows.data_ptr(), r.tiles, r.top if gather else 0, N, K, _stream())
 
 
-def activate(gu, act, limit, alpha):
-    """gu f32 [pairs, 2 F] (gate | up) -> act [pairs, F] = g sigmoid(alpha g) (u + 1) with g = min(gate,
-    limit), u = clamp(up, -limit, limit)."""
+def activate(gu, act, limit, alpha, shift=1.0):
+    """gu f32 [pairs, 2 F] (gate | up) -> act [pairs, F] = g sigmoid(alpha g) (u + shift) with g = min(gate,
+    limit), u = clamp(up, -limit, limit). (limit inf, alpha 1, shift 0: silu(gate) up.)"""
     rows, two_f = gu.shape
     _check(gu, "gate_up", torch.float32, (rows, two_f))
     if two_f % 2:
         raise BackendError("moe activation: the input's width must be even")
     _check(act, "act", None, (rows, two_f // 2))
     lib.call("moe", "hb_moe_activate", gu.data_ptr(), act.data_ptr(), dtype_code(act), rows, two_f // 2, float(limit),
-             float(alpha), _stream())
+             float(alpha), float(shift), _stream())
 
 
-def combine(y, routing, x):
-    """x[t] += sum_j weight[t, j] * y[row of pair (t, j)]; y f32 [pairs, H], x f32 [T, H]."""
+def combine(y, routing, x, shared=None, gate=None):
+    """x[t] += sum_j weight[t, j] * y[row of pair (t, j)]; y f32 [pairs, H], x f32 [T, H].
+    shared f32 [T, H] with gate = (f32 [T, ld], column): x[t] += sigmoid(gate[t, column]) * shared[t] as well."""
     r = routing
     H = x.shape[1]
+    shared_ptr = gate_ptr = None
+    gate_ld = 0
+    if shared is not None:
+        rows, column = gate
+        _check(shared, "shared", torch.float32, (r.T, H))
+        _check(rows, "gate", torch.float32, (r.T, None))
+        gate_ld = rows.shape[1]
+        if not 0 <= column < gate_ld:
+            raise BackendError("moe combine: the gate's column lies outside its rows")
+        shared_ptr, gate_ptr = shared.data_ptr(), rows.data_ptr() + 4 * column
     _check(y, "y", torch.float32, (r.T * r.top, H))
     _check(x, "x", torch.float32, (r.T, H))
     lib.call("moe", "hb_moe_combine", y.data_ptr(), r.weight.data_ptr(), r.row_of.data_ptr(), x.data_ptr(), r.T,
-             r.top, H, _stream())
+             r.top, H, shared_ptr, gate_ptr, gate_ld, _stream())
 
 
 EPI_F32, EPI_BF16, EPI_GLU = 0, 1, 2
@@ -109,12 +131,12 @@ def pack_grouped(w):
 
 
 def grouped_mfma(a, lda, a_group_off, w, c, ldc, c_group_off, epi, routing=None, gather=False, M=0, limit=0.0,
-                 alpha=0.0):
+                 alpha=0.0, shift=1.0):
     """Group g: C[rows, g * c_group_off + n] = sum_k A[src(row), g * a_group_off + k] * w[g][n, k], bfloat16
     operands, float32 sums; w as pack_grouped gives it. With `routing` the rows are the (token, expert) pairs in their experts' order
     (gather: A's rows are the tokens'); without, every group takes the same M rows. epi: EPI_F32 / EPI_BF16
     store C in that type; EPI_GLU: w[g] is [2 F, K] (gate rows, then up rows) and C bfloat16 [*, F] receives
-    the experts' activation with `limit` and `alpha`."""
+    the experts' activation with `limit`, `alpha` and `shift` (see activate)."""
     G, N, K = w.shape
     _check(a, "a", torch.bfloat16)
     _check(w, "w", torch.bfloat16, (G, N, K))
@@ -138,4 +160,4 @@ def grouped_mfma(a, lda, a_group_off, w, c, ldc, c_group_off, epi, routing=None,
             (rows_c - 1) * ldc + (G - 1) * c_group_off + out_cols > c.numel():
         raise BackendError("grouped product: an operand does not hold every row that is addressed")
     lib.call("moe", "hb_grouped_mfma", a.data_ptr(), lda, a_group_off, w.data_ptr(), N, K, c.data_ptr(), ldc,
-             c_group_off, epi, *lists, float(limit), float(alpha), 1 if few else 0, _stream())
+             c_group_off, epi, *lists, float(limit), float(alpha), float(shift), 1 if few else 0, _stream())

@@ -138,16 +138,28 @@ def rope_write_adds_slices(T, hd, rot_dims, dtype, write_kv, has_rotation):
             and (not has_rotation or rot_dims == hd))
 
 
+def query_temperature_args(q_temp):
+    """(coef, every) as the kernels take them; None: (0, 0), no factor."""
+    if q_temp is None:
+        return 0.0, 0
+    coef, every = float(q_temp[0]), int(q_temp[1])
+    if every <= 0:
+        raise BackendError("a query's factor grows every so many positions: that number must be positive")
+    return coef, every
+
+
 def qk_norm_rope_write(qkv, q_norm_w, k_norm_w, cos, sin, rot_dims, meta, cache, q_out, nq, nkv, hd, eps,
-                       write_kv=True, qkv_slices=None):
+                       write_kv=True, qkv_slices=None, q_temp=None):
     """Per-head norm (if weights given), rotation (if tables given), q to q_out, k / v to the pages.
 
     qkv f32 [T, (nq + 2 nkv) hd] (query heads only when write_kv is false); cos / sin f32 [max_pos, rot_dims / 2]; q_out [T, nq hd] in the
     cache's dtype; cache.k / cache.v [pages, nkv, page_size, hd].
     qkv_slices = (slices, pointer, floats between two), as kernels.mfma.gemm(..., defer_slices=True)
     returns it: the projection's sums still lie in that many slices (see rope_write_adds_slices),
-    and qkv itself is not read.
+    and qkv itself is not read. q_temp = (coef, every): a query at position p is multiplied by
+    1 + coef ln(floor((p + 1) / every) + 1) after its norm and rotation.
     """
+    coef, every = query_temperature_args(q_temp)
     T = qkv.shape[0]
     _check(qkv, "qkv", torch.float32, (T, (nq + (2 * nkv if write_kv else 0)) * hd))
     _check_paged(meta, cache, T)
@@ -172,7 +184,7 @@ def qk_norm_rope_write(qkv, q_norm_w, k_norm_w, cos, sin, rot_dims, meta, cache,
              meta.seq_of.data_ptr(), meta.slots.data_ptr(), cache.page_table.data_ptr(),
              cache.page_table.shape[1], cache.page_size, q_out.data_ptr(), cache.k.data_ptr(),
              cache.v.data_ptr(), dtype_code(q_out), T, nq, nkv, hd, float(eps), 1 if write_kv else 0,
-             n_slices, stride, _stream())
+             n_slices, stride, coef, every, _stream())
 
 
 def attention_plain(q, meta, cache, out, nq, nkv, hd, scale, window):
@@ -403,3 +415,48 @@ def layernorm_free_sum(x, delta, mult):
     _check(delta, "delta", torch.float32, tuple(x.shape))
     lib.call("elementwise", "hb_layernorm", x.data_ptr(), delta.data_ptr(), float(mult), None, None, F32, None,
              x.shape[0], x.shape[1], 0.0, _stream())
+
+
+def postnorm(src, weight, x, y, eps, alpha_next, acc=None):
+    """Between two parts of a layer whose norm comes after the sum: x = src / rms(src) * weight (weight
+    None: x = src), y = x in y's dtype, acc = alpha_next * x (alpha_next 0: none). src f32 [T, H]; x f32
+    [T, H] or None; y [T, H] or None; acc f32 [T, H], src itself if not given."""
+    _check(src, "src", torch.float32, (None, None))
+    T, H = src.shape
+    if acc is None:
+        acc = src
+    else:
+        _check(acc, "acc", torch.float32, (T, H))
+    if weight is not None:
+        _check(weight, "weight", torch.float32, (H,))
+    for t, name in ((x, "x"), (y, "y")):
+        if t is not None:
+            _check(t, name, torch.float32 if name == "x" else None, (T, H))
+            if t.data_ptr() in (src.data_ptr(), acc.data_ptr()):
+                raise BackendError(f"postnorm: {name} must be other rows than the source and the sum")
+    lib.call("elementwise", "hb_postnorm", src.data_ptr(), _ptr(weight), _ptr(x), _ptr(y),
+             dtype_code(y) if y is not None else F32, acc.data_ptr(), T, H, float(eps), float(alpha_next),
+             _stream())
+
+
+def relu_squared(z, out):
+    """out = max(z, 0)^2; z f32, out of the same shape in any storage type."""
+    _check(z, "z", torch.float32)
+    _check(out, "out", None, tuple(z.shape))
+    lib.call("elementwise", "hb_relu_squared", z.data_ptr(), out.data_ptr(), dtype_code(out), z.numel(), _stream())
+
+
+def gemm_plain_columns(a, col0, K, w, c, accumulate=False):
+    """c[M, N] (+)= a[:, col0:col0 + K] @ w[N, K]^T in float32 arithmetic: the product of some columns of
+    wider rows, read where they lie."""
+    _check(a, "a", None, (None, None))
+    _check(w, "w", None, (None, K))
+    M, lda = a.shape
+    N = w.shape[0]
+    if col0 < 0 or col0 + K > lda:
+        raise BackendError(f"gemm: columns [{col0}, {col0 + K}) of rows of {lda}")
+    _check(c, "c", None, (M, N))
+    if accumulate and c.dtype != torch.float32:
+        raise BackendError("gemm: accumulation needs a float32 output")
+    lib.call("gemm_plain", "hb_gemm_plain", a.data_ptr() + col0 * a.element_size(), dtype_code(a), w.data_ptr(),
+             dtype_code(w), c.data_ptr(), dtype_code(c), M, N, K, lda, K, N, 1 if accumulate else 0, _stream())

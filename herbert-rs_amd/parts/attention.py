@@ -10,7 +10,18 @@ query heads sharing a kv head (decode.rs:131-140), causal by count
 (prefill/kernel_f32.rs:65-67), output projection added to the residual
 (prefill/mod.rs:293, bc/generic_layer.rs:1234-1236).
 A window (keys of the last `window` positions only) is a parameter that the
-reference does not have.
+reference does not have. Nor are these: values of another size than the keys
+(`value_dim`), a per-head norm without weights (`qk_norm="plain"`), and a query
+that grows with the logarithm of its position (`q_temp=(coef, every)`: times
+1 + coef ln(floor((p + 1) / every) + 1) at position p, after norm and rotation).
+
+The kernels keep one head size for queries, keys and values. Where a model's
+key and value sizes differ, or where the matrix cores (heads of 32, 64, 128)
+would otherwise refuse a head, the part runs them at a larger size whose
+further entries are zeros: zero rows of the projections, zero columns of the
+output projection. Zeros change no score and no weighted sum; the norm's mean
+over the true size d instead of the kept size s is the same as a mean over s
+with eps d / s, times sqrt(d / s) a vector, so the score scale takes d / s.
 """
 import math
 
@@ -29,20 +40,29 @@ class Attention(Part):
     graph_safe = True
 
     def __init__(self, hidden_size, num_heads, num_kv_heads, head_dim, eps, position, names,
-                 qk_norm=True, window=None, scale=None, shared=None, reads_cache_only=False):
-        """names: dict with q, k, v, o (and q_norm, k_norm when qk_norm) -> tensor names.
+                 qk_norm=True, window=None, scale=None, shared=None, reads_cache_only=False,
+                 value_dim=None, q_temp=None):
+        """names: dict with q, k, v, o (and q_norm, k_norm when qk_norm is True) -> tensor names.
+        qk_norm: True (a weight [head_dim] each for queries and keys), "plain" (no weights) or False.
         reads_cache_only: the part has no k / v projections and attends over a cache that
         another entry of the schedule fills."""
         if num_heads % num_kv_heads:
             raise ValueError("num_heads must be divisible by num_kv_heads")
+        if qk_norm not in (True, False, "plain"):
+            raise ValueError(f"qk_norm is True, False or 'plain', not {qk_norm!r}")
         self.hidden_size = int(hidden_size)
         self.nq = int(num_heads)
         self.nkv = int(num_kv_heads)
-        self.hd = int(head_dim)
+        self.dim = int(head_dim)                                       # of a query and a key, as stored
+        self.vdim = int(value_dim) if value_dim else self.dim          # of a value, as stored
+        self.hd = max(self.dim, self.vdim)                             # as kept (load may choose a larger one)
         self.eps = float(eps)
-        self.qk_norm = bool(qk_norm)
+        self.qk_norm = qk_norm
         self.window = int(window) if window else None
-        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.hd)
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.dim)
+        self.q_temp = None if q_temp is None else (float(q_temp[0]), int(q_temp[1]))
+        if self.q_temp is not None and self.q_temp[1] <= 0:
+            raise ValueError("q_temp = (coef, every) with every a positive number of positions")
         self.names = dict(names)
         self.reads_cache_only = bool(reads_cache_only)
         self.position = shared.position(position)
@@ -56,18 +76,55 @@ class Attention(Part):
     def kv_dim(self):
         return self.nkv * self.hd
 
+    # what the kernels are told where the kept size is larger than the keys' own (see the module's text)
+    @property
+    def kernel_eps(self):
+        return self.eps * self.dim / self.hd
+
+    @property
+    def kernel_scale(self):
+        return self.scale * self.dim / self.hd if self.qk_norm else self.scale
+
     def tensor_needs(self):
-        n = self.names
-        needs = {n["q"]: TensorNeed((self.q_dim, self.hidden_size)),
-                 n["o"]: TensorNeed((self.hidden_size, self.q_dim))}
+        n, W = self.names, self.hidden_size
+        needs = {n["q"]: TensorNeed((self.nq * self.dim, W)),
+                 n["o"]: TensorNeed((W, self.nq * self.vdim))}
         if not self.reads_cache_only:
-            needs[n["k"]] = TensorNeed((self.kv_dim, self.hidden_size))
-            needs[n["v"]] = TensorNeed((self.kv_dim, self.hidden_size))
-        if self.qk_norm:
-            needs[n["q_norm"]] = TensorNeed((self.hd,), "scale")
+            needs[n["k"]] = TensorNeed((self.nkv * self.dim, W))
+            needs[n["v"]] = TensorNeed((self.nkv * self.vdim, W))
+        if self.qk_norm is True:
+            needs[n["q_norm"]] = TensorNeed((self.dim,), "scale")
             if not self.reads_cache_only:
-                needs[n["k_norm"]] = TensorNeed((self.hd,), "scale")
+                needs[n["k_norm"]] = TensorNeed((self.dim,), "scale")
         return needs
+
+    def _kept_size(self, rt):
+        """The head size the kernels run at: the larger of keys and values, and in bfloat16 the next size
+        that the matrix cores take, unless the rotation or a cache that another entry fills forbids it."""
+        size = max(self.dim, self.vdim)
+        if self.position.rotation() is not None or self.reads_cache_only:
+            if self.vdim != self.dim:
+                raise ValueError("values of another size than the keys go with no rotation and a cache of the part's own")
+            return size
+        if rt.dtype == torch.bfloat16:
+            for takes in mfma.ATTENTION_HEAD_DIMS:
+                if size <= takes:
+                    return takes
+        return size
+
+    @staticmethod
+    def _heads_padded(w, heads, size, kept, rows=True):
+        """[heads x size, W] -> [heads x kept, W] with zero rows behind every head (rows False: the same
+        for the columns of [W, heads x size])."""
+        if size == kept:
+            return w
+        if rows:
+            out = w.new_zeros((heads, kept, w.shape[1]))
+            out[:, :size] = w.view(heads, size, w.shape[1])
+            return out.view(heads * kept, w.shape[1])
+        out = w.new_zeros((w.shape[0], heads, kept))
+        out[:, :, :size] = w.view(w.shape[0], heads, size)
+        return out.view(w.shape[0], heads * kept)
 
     def cache_need(self):
         if self.reads_cache_only:
@@ -76,16 +133,22 @@ class Attention(Part):
 
     def load(self, tensors, rt):
         n = self.names
-        rows = [tensors[n["q"]]]
+        self.hd = kept = self._kept_size(rt)
+        rows = [self._heads_padded(tensors[n["q"]].to(rt.device), self.nq, self.dim, kept)]
         if not self.reads_cache_only:
-            rows += [tensors[n["k"]], tensors[n["v"]]]
+            rows += [self._heads_padded(tensors[n["k"]].to(rt.device), self.nkv, self.dim, kept),
+                     self._heads_padded(tensors[n["v"]].to(rt.device), self.nkv, self.vdim, kept)]
         # one fused projection [q rows | k rows | v rows]: the activations are read once
-        self.qkv = Linear(rt.weight(torch.cat([r.to(rt.device) for r in rows], 0)), scratch=rt.scratch)
-        self.o = Linear(rt.weight(tensors[n["o"]]), scratch=rt.scratch)
-        if self.qk_norm:
-            self.q_norm_w = rt.weight(tensors[n["q_norm"]], matrix=False)
+        self.qkv = Linear(rt.weight(torch.cat(rows, 0)), scratch=rt.scratch)
+        self.o = Linear(rt.weight(self._heads_padded(tensors[n["o"]].to(rt.device), self.nq, self.vdim, kept, rows=False)),
+                        scratch=rt.scratch)
+        if self.qk_norm is True:
+            pad = lambda w: torch.nn.functional.pad(w, (0, kept - self.dim), value=1.0).contiguous()
+            self.q_norm_w = pad(rt.weight(tensors[n["q_norm"]], matrix=False))
             if not self.reads_cache_only:
-                self.k_norm_w = rt.weight(tensors[n["k_norm"]], matrix=False)
+                self.k_norm_w = pad(rt.weight(tensors[n["k_norm"]], matrix=False))
+        elif self.qk_norm == "plain":
+            self.q_norm_w = self.k_norm_w = torch.ones(kept, dtype=torch.float32, device=rt.device)
 
     def forward_from_residual(self, ctx, x, norm):
         """With few rows and bfloat16 weights no norm kernel runs: the projection takes what the
@@ -113,11 +176,12 @@ class Attention(Part):
         rot = self.position.rotation()
         cos, sin, rot_dims = rot if rot is not None else (None, None, 0)
         if write_kv and fused_norm is None and row_scale is None and rt.dtype == torch.bfloat16:
-            if mfma.gemm_qkv_fusable(y, self.qkv.weight, ctx.meta, kv, self.nq, self.nkv, self.hd, rot_dims):
+            if self.q_temp is None and mfma.gemm_qkv_fusable(y, self.qkv.weight, ctx.meta, kv, self.nq, self.nkv,
+                                                             self.hd, rot_dims):
                 # a long prompt: the projection norms, rotates and writes the cache in its epilogue
                 q = rt.buffer("q", (T, self.q_dim))
                 mfma.gemm_qkv(y, self.qkv.weight, self.qkv.packed, self.q_norm_w, self.k_norm_w, cos, sin, ctx.meta,
-                              kv, q, self.nq, self.nkv, self.hd, self.eps)
+                              kv, q, self.nq, self.nkv, self.hd, self.kernel_eps)
                 attn = rt.buffer("attn", (T, self.q_dim))
                 self.attend(ctx, q, kv, attn)
                 self.project_out(ctx, attn, x)
@@ -139,20 +203,21 @@ class Attention(Part):
         if fused_decode:
             # one token a sequence: norm, rotation, cache write and attention in one kernel
             mfma.attention_decode_fused(qkv, self.q_norm_w, self.k_norm_w, cos, sin, ctx.meta, kv, attn,
-                                        self.nq, self.nkv, self.hd, self.eps, self.scale, self.window,
-                                        qkv_slices=slices, scratch=rt.scratch)
+                                        self.nq, self.nkv, self.hd, self.kernel_eps, self.kernel_scale, self.window,
+                                        qkv_slices=slices, scratch=rt.scratch, q_temp=self.q_temp)
             self.project_out(ctx, attn, x)
             return
         q = rt.buffer("q", (T, self.q_dim))
         ops.qk_norm_rope_write(qkv, self.q_norm_w, self.k_norm_w, cos, sin, rot_dims, ctx.meta, kv, q,
-                               self.nq, self.nkv, self.hd, self.eps, write_kv=write_kv, qkv_slices=slices)
+                               self.nq, self.nkv, self.hd, self.kernel_eps, write_kv=write_kv, qkv_slices=slices,
+                               q_temp=self.q_temp)
         self.attend(ctx, q, kv, attn)
         self.project_out(ctx, attn, x)
 
     def attend(self, ctx, q, kv, out):
         if q.dtype == torch.bfloat16:
             if mfma.attention_supported(q, kv, self.nq, self.nkv, self.hd):
-                mfma.attention(q, ctx.meta, kv, out, self.nq, self.nkv, self.hd, self.scale, self.window,
+                mfma.attention(q, ctx.meta, kv, out, self.nq, self.nkv, self.hd, self.kernel_scale, self.window,
                                scratch=ctx.rt.scratch)
                 return
-        ops.attention_plain(q, ctx.meta, kv, out, self.nq, self.nkv, self.hd, self.scale, self.window)
+        ops.attention_plain(q, ctx.meta, kv, out, self.nq, self.nkv, self.hd, self.kernel_scale, self.window)

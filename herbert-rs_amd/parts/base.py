@@ -8,6 +8,8 @@ in the compute dtype; T counts the tokens of the step, packed over sequences):
   feed_forward  forward(ctx, y, x)                         adds its output to x
   position      rotation() -> (cos, sin, rotary_dims) or None, tables on the GPU
   block         forward(ctx, x)                            runs one layer on x in place
+                (a part of a block may be given rows that are not a norm of x, and other rows to add to
+                than x: "postnorm" hands its parts x itself and rows that already hold alpha x)
   embedding     forward(ctx, token_ids) -> x
   head          forward(ctx, x, rows) -> float32 logits [len(rows), vocab]
 
@@ -154,6 +156,9 @@ class StepContext:
     pending_sum: Any = None
     # rows that hold nothing yet: a part whose last product is to add to exactly these rows stores there instead
     fresh_rows: Any = None
+    # (x's address, alpha): a block whose norm comes after the sum has left, for the next such block, the
+    # rows that its first part reads and alpha times x where that part adds
+    pending_post: Any = None
 
     def adds_to(self, x):
         """False if x are the context's fresh rows (the part's product stores), True if it has to add."""

@@ -3,6 +3,9 @@
 "parallel": with h = norm(x), x += mult * (mixer(h) + feed_forward(h)): one norm, both parts read it,
 and their sum joins the residual stream times a constant.
 
+"postnorm": x <- norm_post_mixer(alpha x + mixer(x)); x <- norm_post_ff(alpha x + feed_forward(x)): the parts
+read x itself, and each norm comes after its sum.
+
 "prenorm": x += mixer(norm_input(x)); x += feed_forward(norm_post_mixer(x)), the
 arrangement of the reference's two-norm layer
 (crates/backends/backend_common/src/generic_layer.rs:1149-1151, 1234-1236,
@@ -118,3 +121,57 @@ class ParallelBlock(Part):
             ctx.pending_sum = (x, total, self.mult)
         else:
             ops.layernorm_free_sum(x, total, self.mult)
+
+
+@register("block", "postnorm")
+class PostNormBlock(Part):
+    """x <- norm_post_mixer(alpha x + mixer(x)), then x <- norm_post_ff(alpha x + feed_forward(x)) (the second
+    step only where the layer has a feed-forward). The parts read x itself, in the compute dtype, and add
+    their outputs, as they always do, to float32 rows: rows that already hold alpha x. One kernel between
+    two parts norms those rows into x, writes the copy that the next part reads and alpha x where it adds;
+    the one after a layer's last part does so for the next layer too, if that is such a block."""
+    graph_safe = True
+
+    norm_roles = ("post_mixer", "post_ff")
+
+    def __init__(self, mixer, feed_forward, norms, alpha=1.0):
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.norms = norms
+        self.alpha = float(alpha)
+        missing = [r for r in self.norm_roles[:1 if feed_forward is None else 2] if r not in norms]
+        if missing:
+            raise ValueError(f"postnorm block needs norms {missing}")
+        if self.alpha == 0.0:
+            raise ValueError("postnorm block: alpha must not be zero")
+        for role in self.norm_roles:
+            if role in norms and not getattr(norms[role], "hands_on", False):
+                raise ValueError("postnorm block: its norms are of the form x * w / rms(x)")
+
+    def parts(self):
+        parts = [self.mixer, self.norms["post_mixer"]]
+        if self.feed_forward is not None:
+            parts += [self.feed_forward, self.norms["post_ff"]]
+        return parts
+
+    def forward(self, ctx, x):
+        rt = ctx.rt
+        shape = tuple(x.shape)
+        acc = rt.buffer("postnorm_sum", shape, torch.float32)
+        y = None if rt.exact else rt.buffer("postnorm_rows", shape)       # (float32: the parts read x itself)
+        pending, ctx.pending_post = ctx.pending_post, None
+        if pending != (x.data_ptr(), self.alpha):
+            ops.postnorm(x, None, None, y, 0.0, self.alpha, acc=acc)
+        nxt = ctx.next_block
+        alpha_after = nxt.alpha if isinstance(nxt, PostNormBlock) else 0.0
+        steps = [(self.mixer, self.norms["post_mixer"])]
+        if self.feed_forward is not None:
+            steps.append((self.feed_forward, self.norms["post_ff"]))
+        for i, (part, norm) in enumerate(steps):
+            ctx.handed = ctx.norm_ahead = ctx.left = ctx.fresh_rows = None
+            part.forward(ctx, x if y is None else y, acc)
+            last = i + 1 == len(steps)
+            ops.postnorm(acc, norm.w, x, None if last and alpha_after == 0.0 else y, norm.eps,
+                         alpha_after if last else self.alpha)
+        if alpha_after != 0.0:
+            ctx.pending_post = (x.data_ptr(), alpha_after)

@@ -11,11 +11,17 @@ its root mean square over vdim, multiplied by a weight [vdim] that the heads sha
 silu(W_g h), and goes through W_o. The recurrence and everything that enters it but the
 projections is float32 in either mode. What a sequence carries from step to step: S, and the last
 K - 1 inputs of the convolution.
+
+Variants, each a parameter: `decay="channel"`: g is a factor a head and key channel (it scales the rows
+of S), g = exp(-exp(A_log[h]) softplus(a + dt_bias)) with a and dt_bias of size heads x dim; `low_rank`:
+the decay's pre-activation a and the gate's are each two products, W_2 (W_1 h), through a narrow
+middle (names a1, a2, g1, g2 in place of a, g); `gate="sigmoid"`: the output is gated by
+sigmoid(.) instead of silu(.).
 """
 import torch
 
 from ..cache import StateNeed
-from ..kernels import recurrent
+from ..kernels import ops, recurrent
 from ..weights import TensorNeed
 from .base import Part
 from .linear import Linear
@@ -34,14 +40,30 @@ def _rate_init(shape, gen, device, std, norm_std):
     return 0.5 * torch.randn(shape, generator=gen, device=device, dtype=torch.float32)
 
 
+def _second_init(shape, gen, device, std, norm_std):
+    """The second of two products through a narrow middle: drawn so that the pair's output is about as
+    large as one full-width product's with the model's deviation would be (the middle's entries are sums
+    of `width` terms of deviation std each; 1 / sqrt(middle) brings their sum back to one entry's size)."""
+    return torch.randn(shape, generator=gen, device=device, dtype=torch.float32) / shape[1] ** 0.5
+
+
 @register("mixer", "gated_delta")
 class GatedDelta(Part):
     graph_safe = True
     stores_fresh_rows = True     # its output projection stores into rows that hold nothing yet (StepContext.adds_to)
 
-    def __init__(self, hidden_size, heads, kv_heads, dim, vdim, conv, eps, names, unit_eps=UNIT_EPS, shared=None):
-        """names: q, k, v, q_conv, k_conv, v_conv, b, a, A_log, dt_bias, g, norm, o -> tensor names.
-        conv: the taps of the convolution (1: none). eps: of the norm a head."""
+    def __init__(self, hidden_size, heads, kv_heads, dim, vdim, conv, eps, names, unit_eps=UNIT_EPS, shared=None,
+                 decay="head", low_rank=None, gate="silu"):
+        """names: q, k, v, q_conv, k_conv, v_conv, b, a, A_log, dt_bias, g, norm, o -> tensor names
+        (with low_rank: a1, a2, g1, g2 in place of a and g).
+        conv: the taps of the convolution (1: none). eps: of the norm a head. decay: "head" or "channel".
+        low_rank: None, or (the middle's size of the decay, of the gate); None for one of them: read from
+        the stored tensor's shape. gate: "silu" or "sigmoid"."""
+        if decay not in ("head", "channel") or gate not in ("silu", "sigmoid"):
+            raise ValueError(f"the delta rule's decay is 'head' or 'channel' and its gate 'silu' or 'sigmoid', "
+                             f"not {decay!r} and {gate!r}")
+        self.decay, self.gate = decay, gate
+        self.low_rank = None if low_rank is None else tuple(low_rank)
         if heads % kv_heads:
             raise ValueError("heads must be divisible by kv_heads")
         self.hidden_size, self.heads, self.kv_heads = int(hidden_size), int(heads), int(kv_heads)
@@ -58,18 +80,34 @@ class GatedDelta(Part):
         """Channels that pass the convolution: queries, keys, values."""
         return 2 * self.kv_heads * self.dim + self.heads * self.vdim
 
+    @property
+    def decay_width(self):
+        """Pre-activations of the decay a token: one a head, or one a head and key channel."""
+        return self.heads * (self.dim if self.decay == "channel" else 1)
+
     def tensor_needs(self):
         n, W = self.names, self.hidden_size
         qk, v = self.kv_heads * self.dim, self.heads * self.vdim
-        return {n["q"]: TensorNeed((qk, W)), n["k"]: TensorNeed((qk, W)), n["v"]: TensorNeed((v, W)),
-                n["q_conv"]: TensorNeed((qk, self.taps), "taps", _taps_init),
-                n["k_conv"]: TensorNeed((qk, self.taps), "taps", _taps_init),
-                n["v_conv"]: TensorNeed((v, self.taps), "taps", _taps_init),
-                n["b"]: TensorNeed((self.heads, W)), n["a"]: TensorNeed((self.heads, W)),
-                n["A_log"]: TensorNeed((self.heads,), "rate", _rate_init),
-                n["dt_bias"]: TensorNeed((self.heads,), "rate", _rate_init),
-                n["g"]: TensorNeed((v, W)), n["norm"]: TensorNeed((self.vdim,), "scale"),
-                n["o"]: TensorNeed((W, v))}
+        needs = {n["q"]: TensorNeed((qk, W)), n["k"]: TensorNeed((qk, W)), n["v"]: TensorNeed((v, W)),
+                 n["q_conv"]: TensorNeed((qk, self.taps), "taps", _taps_init),
+                 n["k_conv"]: TensorNeed((qk, self.taps), "taps", _taps_init),
+                 n["v_conv"]: TensorNeed((v, self.taps), "taps", _taps_init),
+                 n["b"]: TensorNeed((self.heads, W)),
+                 n["A_log"]: TensorNeed((self.heads,), "rate", _rate_init),
+                 n["dt_bias"]: TensorNeed((self.decay_width,), "rate", _rate_init),
+                 n["norm"]: TensorNeed((self.vdim,), "scale"),
+                 n["o"]: TensorNeed((W, v))}
+        if self.low_rank is None:
+            needs[n["a"]] = TensorNeed((self.decay_width, W))
+            needs[n["g"]] = TensorNeed((v, W))
+        else:
+            ra, rg = self.low_rank
+            # (a middle's size that the configuration does not give is whatever the stored tensor has)
+            needs[n["a1"]] = TensorNeed((ra, W))
+            needs[n["a2"]] = TensorNeed((self.decay_width, ra), "matrix", _second_init)
+            needs[n["g1"]] = TensorNeed((rg, W))
+            needs[n["g2"]] = TensorNeed((v, rg), "matrix", _second_init)
+        return needs
 
     def cache_need(self):
         needs = [StateNeed((self.heads, self.dim, self.vdim), torch.float32)]
@@ -80,12 +118,18 @@ class GatedDelta(Part):
     def load(self, tensors, rt):
         n = self.names
         # one projection [q | k | v | g | b | a]: the rows are read once; its float32 sums feed the
-        # convolution, the gate and the recurrence's two scalars a head
-        rows = [tensors[n[k]].to(rt.device) for k in ("q", "k", "v", "g", "b", "a")]
+        # convolution, the gate and the recurrence's two scalars a head (with low_rank, g and a are the
+        # narrow middles, and a second product each widens them)
+        first = ("q", "k", "v", "g", "b", "a") if self.low_rank is None else ("q", "k", "v", "g1", "b", "a1")
+        rows = [tensors[n[k]].to(rt.device) for k in first]
         self.proj = Linear(rt.weight(torch.cat(rows, 0)), scratch=rt.scratch)
-        C, V = self.channels, self.heads * self.vdim
-        self.g_off, self.b_off, self.a_off = C, C + V, C + V + self.heads
-        self.width = C + V + 2 * self.heads
+        C = self.channels
+        g_width, a_width = rows[3].shape[0], rows[5].shape[0]
+        self.g_off, self.b_off, self.a_off = C, C + g_width, C + g_width + self.heads
+        self.width = C + g_width + self.heads + a_width
+        self.g_width, self.a_width = g_width, a_width
+        if self.low_rank is not None:
+            self.a2, self.g2 = rt.weight(tensors[n["a2"]]), rt.weight(tensors[n["g2"]])
         self.conv_w = torch.cat([rt.weight(tensors[n[k]], matrix=False) for k in ("q_conv", "k_conv", "v_conv")], 0).contiguous()
         self.a_log = rt.weight(tensors[n["A_log"]], matrix=False)
         self.dt_bias = rt.weight(tensors[n["dt_bias"]], matrix=False)
@@ -104,10 +148,24 @@ class GatedDelta(Part):
         recurrent.conv_silu(proj, self.conv_w, conv_state, ctx.meta, qkv, 2 * self.kv_heads, self.dim, self.kv_heads,
                             self.dim ** -0.5, self.unit_eps, self.heads, self.vdim)
         o = rt.buffer("delta_o", (T, self.heads * self.vdim), torch.float32)
-        recurrent.gated_delta(qkv, proj, self.b_off, self.a_off, self.a_log, self.dt_bias, state, ctx.meta, o,
-                              self.kv_heads, self.heads, self.dim, self.vdim)
+        gate_rows, gate_off, decay_rows, decay_off = proj, self.g_off, proj, self.a_off
+        if self.low_rank is not None:
+            # the second products, float32 sums of the float32 middles
+            gate_rows, gate_off = rt.buffer("delta_gate", (T, self.heads * self.vdim), torch.float32), 0
+            ops.gemm_plain_columns(proj, self.g_off, self.g_width, self.g2, gate_rows)
+            decay_rows, decay_off = rt.buffer("delta_decay", (T, self.decay_width), torch.float32), 0
+            ops.gemm_plain_columns(proj, self.a_off, self.a_width, self.a2, decay_rows)
+        if self.decay == "channel":
+            factors = rt.buffer("delta_decay", (T, self.decay_width), torch.float32)
+            recurrent.channel_decay(decay_rows, decay_off, self.a_log, self.dt_bias, factors, self.heads, self.dim)
+            recurrent.gated_delta(qkv, proj, self.b_off, 0, None, None, state, ctx.meta, o,
+                                  self.kv_heads, self.heads, self.dim, self.vdim, decay=factors)
+        else:
+            recurrent.gated_delta(qkv, decay_rows, self.b_off, decay_off, self.a_log, self.dt_bias, state, ctx.meta, o,
+                                  self.kv_heads, self.heads, self.dim, self.vdim)
         gated = rt.buffer("delta_gated", (T, self.heads * self.vdim))
-        recurrent.gated_head_norm(o, proj, self.g_off, self.norm_w, gated, self.heads, self.vdim, self.eps)
+        recurrent.gated_head_norm(o, gate_rows, gate_off, self.norm_w, gated, self.heads, self.vdim, self.eps,
+                                  gate=self.gate)
         adds = ctx.adds_to(x)
         left = ctx.leave_norm(self.o, x) if adds else None
         self.o.forward(gated, x, accumulate=adds, leave=None if left is None else left.leave())

@@ -1,6 +1,7 @@
 """The two ends of a model: the embedding table and the output head.
 
-Embedding without multiplier (crates/backends/backend_common/src/generic_model.rs:104-111);
+Embedding without multiplier (crates/backends/backend_common/src/generic_model.rs:104-111; `scale` is a
+parameter for families that have one);
 the head is the final norm of the wanted rows only and a product with
 lm_head, or with the embedding table when the two are tied
 (generic_model.rs:266-283; loader_common.rs:1851-1872).
@@ -18,9 +19,11 @@ from .registry import build, register
 class TokenEmbedding(Part):
     graph_safe = True
 
-    def __init__(self, vocab_size, hidden_size, weight, shared=None, norm=None):
+    def __init__(self, vocab_size, hidden_size, weight, shared=None, norm=None, scale=None):
         """norm: a PartSpec of a norm that the gathered rows pass before they are the residual stream
-        (it must offer forward_in_place), or None."""
+        (it must offer forward_in_place), or None. scale: the gathered rows times this constant (a head
+        tied to the table uses the table as it is)."""
+        self.scale = None if scale is None or float(scale) == 1.0 else float(scale)
         self.vocab_size = int(vocab_size)
         self.hidden_size = int(hidden_size)
         self.weight_name = weight
@@ -44,6 +47,8 @@ class TokenEmbedding(Part):
     def forward(self, ctx, token_ids):
         x = ctx.rt.buffer("residual", (token_ids.shape[0], self.hidden_size), torch.float32)
         ops.embed(token_ids, self.table, x, packed=self.linear.packed)
+        if self.scale is not None:
+            ops.scale(x, self.scale)
         if self.norm is not None:
             self.norm.forward_in_place(ctx, x)
         return x

@@ -1,4 +1,4 @@
-"""Dense gated feed-forward: down(silu(gate(y)) * up(y)), no biases.
+"""Dense feed-forwards without biases. "swiglu": down(silu(gate(y)) * up(y)). "squared_relu": down(max(up(y), 0)^2).
 
 crates/backends/backend_common/src/generic_mlp.rs:83-96 and kernels.rs:676-687
 of the reference; gate and up are one fused matrix here so that the activations
@@ -71,5 +71,38 @@ class SwiGLU(Part):
             gu = rt.buffer("gate_up", (T, 2 * self.intermediate_size), torch.float32)
             self.gate_up.forward(y, gu)
             ops.swiglu(gu, act)
+        left = ctx.leave_norm(self.down, x)
+        self.down.forward(act, x, accumulate=True, leave=None if left is None else left.leave())
+
+
+@register("feed_forward", "squared_relu")
+class SquaredRelu(Part):
+    """down(max(up(y), 0)^2): two matrices, the activation on the first product's float32 sums."""
+    graph_safe = True
+
+    def __init__(self, hidden_size, intermediate_size, names, shared=None):
+        """names: dict with up, down -> tensor names."""
+        self.hidden_size = int(hidden_size)
+        self.intermediate_size = int(intermediate_size)
+        self.names = dict(names)
+        self.up = self.down = None
+
+    def tensor_needs(self):
+        n = self.names
+        return {n["up"]: TensorNeed((self.intermediate_size, self.hidden_size)),
+                n["down"]: TensorNeed((self.hidden_size, self.intermediate_size))}
+
+    def load(self, tensors, rt):
+        n = self.names
+        self.up = Linear(rt.weight(tensors[n["up"]]), scratch=rt.scratch)
+        self.down = Linear(rt.weight(tensors[n["down"]]), scratch=rt.scratch)
+
+    def forward(self, ctx, y, x):
+        rt = ctx.rt
+        T = x.shape[0]
+        z = rt.buffer("ff_up", (T, self.intermediate_size), torch.float32)
+        self.up.forward(y, z)
+        act = rt.buffer("act", (T, self.intermediate_size))
+        ops.relu_squared(z, act)
         left = ctx.leave_norm(self.down, x)
         self.down.forward(act, x, accumulate=True, leave=None if left is None else left.leave())

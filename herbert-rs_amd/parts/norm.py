@@ -1,9 +1,16 @@
 """Norms of the residual stream. RMSNorm as the reference computes it (crates/backends/backend_common/src/kernels.rs:54-64):
-y = x / sqrt(mean(x^2) + eps) * w, the weight used as stored (not 1 + w)."""
+y = x / sqrt(mean(x^2) + eps) * w, the weight used as stored (not 1 + w). A family whose weights are
+stored around zero gives `offset` 1: the kernels then see offset + w."""
 from ..kernels import ops
 from ..weights import TensorNeed
 from .base import Part
 from .registry import register
+
+
+def _around_zero(shape, gen, device, std, norm_std):
+    """A random model's weights of a norm that adds its offset itself."""
+    import torch
+    return norm_std * torch.randn(shape, generator=gen, device=device, dtype=torch.float32)
 
 
 @register("norm", "rmsnorm")
@@ -11,17 +18,23 @@ class RMSNorm(Part):
     graph_safe = True
     hands_on = True      # y = x * w / rms(x): a product may apply the 1 / rms to its sums instead (NormedRows)
 
-    def __init__(self, size, eps, weight):
+    def __init__(self, size, eps, weight, offset=0.0):
+        """offset: added to the stored weight (1 for weights stored around zero)."""
         self.size = int(size)
         self.eps = float(eps)
         self.weight_name = weight
+        self.offset = float(offset)
         self.w = None
 
     def tensor_needs(self):
+        if self.offset:
+            return {self.weight_name: TensorNeed((self.size,), "scale", _around_zero)}
         return {self.weight_name: TensorNeed((self.size,), "scale")}
 
     def load(self, tensors, rt):
         self.w = rt.weight(tensors[self.weight_name], matrix=False)
+        if self.offset:
+            self.w = (self.w + self.offset).contiguous()
 
     def forward(self, ctx, x, rows=None, name="normed"):
         n = x.shape[0] if rows is None else rows.shape[0]

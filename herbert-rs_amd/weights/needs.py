@@ -14,6 +14,6 @@ class TensorNeed:
     brings its own `init(shape, generator, device, std, norm_std) -> float32 or int32 tensor`;
     nothing else in the library has to know the new kind.
     """
-    shape: Tuple[int, ...]
+    shape: Tuple[Optional[int], ...]      # None: a size that only the stored tensor gives (no random stand-in then)
     role: str = "matrix"
     init: Optional[Callable] = None

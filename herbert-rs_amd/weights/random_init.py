@@ -76,6 +76,9 @@ def random_tensor(name, need, seed, dtype, std=0.02, norm_std=0.0, device="cpu")
     """One tensor for `need`: matrices and tables in `dtype`, scales (norm weights) in float32 then
     `dtype`, integers int32. The need's own initialiser decides if it has one, else its role."""
     init = need.init or ROLE_INITIALISERS.get(need.role)
+    if any(d is None for d in need.shape):
+        raise ConfigError(f"tensor {name}: the configuration leaves a size of {list(need.shape)} to the stored "
+                          "tensor, so no random one can be drawn; name the size in the configuration")
     if init is not None:
         gen = torch.Generator(device=device)
         gen.manual_seed(_tensor_seed(seed, name))

@@ -88,7 +88,9 @@ def read_tensors(folder, needs, device="cpu", name_map=None, strict=False, ignor
                     expected = tuple(needs[name].shape)
                 else:       # the parts' rows one after the other
                     expected = (sum(needs[t].shape[0] for t in targets),) + tuple(needs[targets[0]].shape[1:])
-                if shape != expected:
+                # (a size that the need leaves open, None, is whatever the file has; parts that ask for
+                # several such tensors check that they fit each other when they take them)
+                if len(shape) != len(expected) or any(e is not None and e != s for e, s in zip(expected, shape)):
                     wrong.append(f"{stored}: expected {list(expected)}, got {list(shape)}")
                     for n in (targets or [name]):
                         found[n] = None
