@@ -177,15 +177,24 @@ class ModasunConfig:
             mlp = None
             if entry.get("mlp") is not None:
                 mlp = _mlp(_section(entry, "mlp", where + "."), where + ".mlp")
-            source = Reader(entry).integer("weights_of")
-            if source is not None:
-                if not 0 <= source < i or layers[source].weights_of is not None:
-                    raise ConfigError(f"config.json: {where}.weights_of must name an earlier layer that has tensors "
+            layers.append(ModasunLayer(kind, mixer, mlp, Reader(entry).integer("weights_of")))
+        for i, layer in enumerate(layers):
+            if layer.weights_of is None:
+                continue
+            # the layer whose tensors are run: the end of the chain, if the named layer runs another's itself
+            source, seen = layer.weights_of, {i}
+            while True:
+                if not 0 <= source < len(layers) or source in seen:
+                    raise ConfigError(f"config.json: layers[{i}].weights_of must name another layer that has tensors "
                                       "of its own")
-                theirs = layers[source]
-                if (theirs.type, theirs.mixer, theirs.mlp) != (kind, mixer, mlp):
-                    raise ConfigError(f"config.json: {where} runs the weights of layer {source} but differs from it")
-            layers.append(ModasunLayer(kind, mixer, mlp, source))
+                if layers[source].weights_of is None:
+                    break
+                seen.add(source)
+                source = layers[source].weights_of
+            theirs = layers[source]
+            if (theirs.type, theirs.mixer, theirs.mlp) != (layer.type, layer.mixer, layer.mlp):
+                raise ConfigError(f"config.json: layers[{i}] runs the weights of layer {source} but differs from it")
+            layers[i] = ModasunLayer(layer.type, layer.mixer, layer.mlp, source)
         cfg = ModasunConfig(r.integer("vocab", required=True), r.integer("width", required=True), tuple(layers),
                             _section(raw, "norm", "").number("eps", required=True),
                             r.number("postln_alpha", required=True),

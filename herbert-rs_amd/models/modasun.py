@@ -54,10 +54,9 @@ def _norm(cfg, weight):
 
 
 def build_spec(cfg):
-    layers, schedule, spec_of = [], [], {}
+    layers, spec_of = [], {}
     for i, layer in enumerate(cfg.layers):
         if layer.weights_of is not None:
-            schedule.append(ScheduleEntry(spec_of[layer.weights_of]))
             continue
         mixer = MIXER_SPECS[layer.type](cfg, layer.mixer, f"l{i}.mix.")
         norms = {"post_mixer": _norm(cfg, f"l{i}.norm1")}
@@ -67,7 +66,9 @@ def build_spec(cfg):
             norms["post_ff"] = _norm(cfg, f"l{i}.norm2")
         spec_of[i] = len(layers)
         layers.append(LayerSpec(PartSpec("postnorm", {"alpha": cfg.postln_alpha}), mixer, ffn, norms))
-        schedule.append(ScheduleEntry(spec_of[i]))
+    # every listed layer is one run of the schedule, with a cache entry of its own, whoever's tensors it runs
+    schedule = [ScheduleEntry(spec_of[i if layer.weights_of is None else layer.weights_of])
+                for i, layer in enumerate(cfg.layers)]
     return ModelSpec(
         hidden_size=cfg.hidden_size, vocab_size=cfg.vocab_size, max_positions=cfg.max_position_embeddings,
         embedding=PartSpec("table", {"vocab_size": cfg.vocab_size, "hidden_size": cfg.hidden_size, "weight": "embed",

@@ -29,9 +29,10 @@ F32_ABS = 1e-4
 #  0.0146 and 0.050; "deep": 1 to 36 layers at a quarter of the 8B width, vocabulary 4096: 0.0084 and
 #  0.037 for one layer, 0.0114 and 0.050 for 36: the error hardly grows with depth, and in float32
 #  it goes from 9e-6 for one layer to 1.1e-5 for 36)
-# ("vip": the Vipalorn configurations, whose recurrence, scores and routing stay float32.)
-BF16_REL_L2 = {"vip": 0.03, "A": 0.012, "B": 0.018, "C": 0.018, "D": 0.02, "F": 0.02, "wide": 0.02, "odd": 0.02, "random": 0.02, "long": 0.025, "deep": 0.02}
-BF16_REL_RMS = {"vip": 0.1, "A": 0.04, "B": 0.05, "C": 0.05, "D": 0.05, "F": 0.05, "wide": 0.08, "odd": 0.04, "random": 0.06, "long": 0.08, "deep": 0.08}
+# ("vip": the Vipalorn configurations, whose recurrence, scores and routing stay float32; "mod": the Modasun
+#  configurations, the same and a float32 stream that is normed after every sum.)
+BF16_REL_L2 = {"mod": 0.03, "vip": 0.03, "A": 0.012, "B": 0.018, "C": 0.018, "D": 0.02, "F": 0.02, "wide": 0.02, "odd": 0.02, "random": 0.02, "long": 0.025, "deep": 0.02}
+BF16_REL_RMS = {"mod": 0.1, "vip": 0.1, "A": 0.04, "B": 0.05, "C": 0.05, "D": 0.05, "F": 0.05, "wide": 0.08, "odd": 0.04, "random": 0.06, "long": 0.08, "deep": 0.08}
 
 
 def rel_rms_error(got, ref):
@@ -49,7 +50,7 @@ def close(got, ref, dtype, config, label=None):
         observe(f"float32 {config} {label or ''} abs", err)
         return err <= F32_ABS, err
     ok = rel <= BF16_REL_RMS[config] and rel_l2 <= BF16_REL_L2[config]
-    if ok or config != "vip":        # (of that family's rows a few may be off for a reason that is no rounding: the worst of the others is what counts)
+    if ok or config not in ("vip", "mod"):        # (of that family's rows a few may be off for a reason that is no rounding: the worst of the others is what counts)
         observe(f"bfloat16 {config} {label or ''} max / rms", rel)
         observe(f"bfloat16 {config} {label or ''} rms / rms", rel_l2)
     return ok, max(rel, rel_l2)

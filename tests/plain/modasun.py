@@ -188,9 +188,9 @@ def sub(tensors, prefix):
     return {k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)}
 
 
-def forward(cfg, tensors, tokens, dtype=torch.float32, layers_out=None):
-    """Logits [T, vocab] of one sequence of token ids. layers_out: a list that receives the residual
-    stream after every layer run."""
+def forward(cfg, tensors, tokens, dtype=torch.float32, layers_out=None, rows=None):
+    """Logits [T, vocab] of one sequence of token ids (of the positions `rows` only, if given).
+    layers_out: a list that receives the residual stream after every layer run."""
     t = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in tensors.items()}
     eps, alpha = cfg["norm"]["eps"], cfg["postln_alpha"]
     x = t["embed"][torch.as_tensor(tokens, dtype=torch.long)] * cfg["embedding"]["scale"]
@@ -214,8 +214,20 @@ def forward(cfg, tensors, tokens, dtype=torch.float32, layers_out=None):
             x = offset_norm(alpha * x + ff, t[p + "norm2"], eps)
         if layers_out is not None:
             layers_out.append(x.clone())
+    if rows is not None:
+        x = x[list(rows)]
     x = offset_norm(x, t["final.norm"], eps)
     return linear(x, t["embed"])
+
+
+def greedy(cfg, tensors, prompt, n):
+    """n tokens after the prompt, each the first of the largest logits of the sequence so far."""
+    seq, out = list(prompt), []
+    for _ in range(n):
+        logits = forward(cfg, tensors, seq, rows=[len(seq) - 1])[0]
+        out.append(int(torch.argmax(logits)))
+        seq.append(out[-1])
+    return out
 
 
 def load_folder(folder):
