@@ -20,6 +20,10 @@ cache below the timed steps is filled by real prefill steps of random prompts. A
 step is what the generation loop does for a token: the step function (a HIP-graph replay), the
 greedy choice on the GPU, and the chosen tokens read by the host, which as in that loop reads
 the tokens of a step while the next step, fed from the GPU, already runs.
+
+`--workload vipalorn|modasun --size small|medium|wide` measures one of the other designs instead (random weights at
+sizes that resemble a real model's layers) beside the closest other model at equal size, through the generation
+loop; the default workload and its JSON line stay as they are.
 """
 import argparse
 import json
@@ -165,10 +169,29 @@ def family_configs(size):
     return vip, dense
 
 
-def run_family(args):
-    """Prompt and decode throughput of the Vipalorn design at one size (random weights), beside the dense
-    Qwen3 decoder at equal size, both through the generation loop: prompts of 512 and 2,048 tokens alone,
-    and batches of 1, 8 and 32 sequences of 1,024 prompt tokens decoding `--steps` tokens each."""
+def modasun_configs(size):
+    """(Modasun config dict, Vipalorn config dict) of one size: three delta layers (a decay a key channel, the
+    decay and the gate through middles of a sixteenth of the width) to one attention layer (the softmax
+    attention without rotation), experts chosen within half of four groups beside a shared expert as wide as
+    one expert; and the Vipalorn model of the same width, depth, heads and experts."""
+    W, L, H, D, V, rank, rot, E, top, ff, vocab = FAMILY_SIZES[size]
+    delta = {"type": "channel_delta", "mixer": {"heads": H, "kv_heads": H // 2, "dim": D, "vdim": V, "conv": 4,
+                                                "low_rank": {"decay": W // 16, "gate": W // 16}}}
+    attention = {"type": "attention", "mixer": {"heads": H, "kv_heads": H // 2, "dim": D, "vdim": V, "scale": D ** -0.5,
+                                                "q_temp": {"coef": 0.1, "every": 1024}}}
+    mlp = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": E, "top": top, "groups": {"count": 4, "keep": 2}},
+           "shared": {"ff": ff}}
+    layers = [dict(attention if i % 4 == 3 else delta, mlp=mlp) for i in range(L)]
+    mod = {"architecture": "Modasun", "vocab": vocab, "width": W, "layers": layers, "norm": {"eps": 1e-5},
+           "postln_alpha": 2.0, "embedding": {"scale": 8.0}}
+    return mod, family_configs(size)[0]
+
+
+def run_family(args, names=("vipalorn", "qwen3"), configs=family_configs):
+    """Prompt and decode throughput of a design at one size (random weights) beside the closest other model at
+    equal size (Vipalorn beside the dense Qwen3 decoder, Modasun beside Vipalorn), both through the generation
+    loop: prompts of 512 and 2,048 tokens alone, and batches of 1, 8 and 32 sequences of 1,024 prompt tokens
+    decoding `--steps` tokens each."""
     import torch
     import herbert_rs_amd as hb
     from herbert_rs_amd.config.registry import resolve_architecture
@@ -176,7 +199,7 @@ def run_family(args):
     torch.cuda.set_device(0)
     new = max(args.steps, 8)
     out = {}
-    for name, raw in zip(("vipalorn", "qwen3"), family_configs(args.size)):
+    for name, raw in zip(names, configs(args.size)):
         arch = resolve_architecture(raw)
         cfg = arch.config_class.from_dict(raw)
         t0 = time.time()
@@ -210,15 +233,16 @@ def run_family(args):
         print(f"[bench] {name}: {rec}", file=sys.stderr, flush=True)
         del engine
         torch.cuda.empty_cache()
-    v = out["vipalorn"]
-    return {"metric": f"decode tok/s, Vipalorn design ({args.size} sizes), batch 8, 1024 prompt tokens", "value": v["decode_b8_tok_s"],
+    v = out[names[0]]
+    design = names[0].capitalize()
+    return {"metric": f"decode tok/s, {design} design ({args.size} sizes), batch 8, 1024 prompt tokens", "value": v["decode_b8_tok_s"],
             "unit": "tokens/s", "n_gpus": 1, "steps": new, "warmup": 4, "ms_per_step": v["decode_b8_ms"],
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic: random weights, random token ids",
-            "config": {"model": f"Vipalorn {args.size}", "sizes": dict(zip(
+            "config": {"model": f"{design} {args.size}", "sizes": dict(zip(
                 ("width", "layers", "heads", "key_dim", "value_dim", "latent_rank", "rotated", "experts", "top", "expert_ff", "vocab"),
                 FAMILY_SIZES[args.size])), "global_batch": 8, "parallelism": "single GPU"},
-            "vipalorn": v, "qwen3_equal_size": out["qwen3"]}
+            names[0]: v, names[1] + "_equal_size": out[names[1]]}
 
 
 def main():
@@ -236,9 +260,10 @@ def main():
     ap.add_argument("--no-sweep", action="store_true", help="time the full context only, not 512 and the mean")
     ap.add_argument("--no-long", action="store_true",
                     help="skip the further sizes and lengths (contexts of 16 K and 32 K, batch 128 and 256, long prompts)")
-    ap.add_argument("--size", default="medium", choices=sorted(FAMILY_SIZES), help="layer sizes of --workload vipalorn")
-    ap.add_argument("--workload", default="headline", choices=["headline", "qwen3-1.7b", "qwen3-32b", "vipalorn"],
-                    help="headline: BASELINE.json configs[2]; the others: configs[3] and configs[4]")
+    ap.add_argument("--size", default="medium", choices=sorted(FAMILY_SIZES), help="layer sizes of --workload vipalorn and --workload modasun")
+    ap.add_argument("--workload", default="headline", choices=["headline", "qwen3-1.7b", "qwen3-32b", "vipalorn", "modasun"],
+                    help="headline: BASELINE.json configs[2]; qwen3-*: configs[3] and configs[4]; vipalorn, modasun: "
+                         "that design at --size beside the closest other model at equal size")
     ap.add_argument("--prefill-tokens", type=int, default=2048, help="length of the prompt of the prefill figure")
     ap.add_argument("--prefill-chunk", type=int, default=0,
                     help="feed the prompt of the prefill figure in steps of this many tokens (0: in one step)")
@@ -258,6 +283,9 @@ def main():
 
     if args.workload == "vipalorn":
         print(json.dumps(run_family(args)))
+        return 0
+    if args.workload == "modasun":
+        print(json.dumps(run_family(args, names=("modasun", "vipalorn"), configs=modasun_configs)))
         return 0
     if args.workload != "headline":
         print(json.dumps(run_workload(args, 3 if args.workload == "qwen3-1.7b" else 4,

@@ -3,7 +3,9 @@
 // It is the whole matrix path of the float32 mode and the fallback of the bfloat16
 // mode for shapes its MFMA kernels refuse. Each output is summed over k ascending by
 // one thread with fused multiply-adds, so its value does not depend on M, on the tile
-// it falls in, or on what else is in the batch.
+// it falls in, or on what else is in the batch. (hb_gemm_plain_short_k is the entry for products with a
+// short k: it sends up to 32 float32 rows times bfloat16 rows to gemm_few_rows_kernel, whose four partial
+// sums a column differ from that order by float32 rounding, and everything else here.)
 // In xigh/herbert-rs: crates/backends/backend_bf16/src/kernels.rs:154-164 (float32 sums over k ascending of
 // x[m, k] * float(w[n, k]), no bias); crates/backends/backend_vulkan/shaders/bf16_matmul.comp:31-60.
 #include "common.h"
@@ -95,6 +97,71 @@ static void launch(const void* A, const void* W, void* C, int M, int N, int K, i
             (const TA*)A, (const TW*)W, (TC*)C, M, N, K, lda, ldw, ldc, batch_a, batch_w, batch_c);
 }
 
+
+// Few rows times a matrix of bfloat16 rows with a short k (the second product of a pair through a narrow
+// middle, one token a sequence): the tiled kernel above would run N / 64 workgroups with a barrier every
+// 16 k. Here a wave takes 16 output columns, four lanes a column, each lane a quarter of k in steps of 8
+// (one 16-byte load of the weights' row), for up to 8 rows of A at once, which the wave first copies to
+// LDS so that no load waits for another; the four partial sums meet by two lane exchanges. Float32
+// arithmetic throughout. A's rows and W's rows must be 16-byte aligned, K in steps of 32 up to FEW_ROWS_K.
+#define FEW_ROWS_M 8
+#define FEW_ROWS_K 1024
+__global__ void __launch_bounds__(HB_WAVE)
+gemm_few_rows_kernel(const float* __restrict__ A, const bf16* __restrict__ W, float* __restrict__ C, int M, int N,
+                     int K, int lda, int ldw, int ldc) {
+    __shared__ __attribute__((aligned(16))) float rows_of_a[FEW_ROWS_M * FEW_ROWS_K];
+    const int lane = threadIdx.x;
+    const int n = blockIdx.x * 16 + lane / 4;
+    const int part = lane % 4;
+    const int m0 = blockIdx.y * FEW_ROWS_M;
+    const int rows = M - m0 < FEW_ROWS_M ? M - m0 : FEW_ROWS_M;
+    const int quarter = K / 4;
+    for (int idx = lane; idx < FEW_ROWS_M * quarter; idx += HB_WAVE) {
+        const int i = idx / quarter, f = idx % quarter;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (i < rows) v = *(const float4*)(A + (size_t)(m0 + i) * lda + 4 * f);
+        *(float4*)&rows_of_a[i * K + 4 * f] = v;
+    }
+    __syncthreads();
+    float acc[FEW_ROWS_M];
+#pragma unroll
+    for (int i = 0; i < FEW_ROWS_M; ++i) acc[i] = 0.f;
+    if (n < N) {
+        const bf16* w_row = W + (size_t)n * ldw + part * quarter;
+        const float* a_row = rows_of_a + part * quarter;
+        for (int k = 0; k < quarter; k += 8) {
+            const uint4 packed = *(const uint4*)(w_row + k);
+            float w[8];
+            w[0] = __uint_as_float(packed.x << 16), w[1] = __uint_as_float(packed.x & 0xffff0000u);
+            w[2] = __uint_as_float(packed.y << 16), w[3] = __uint_as_float(packed.y & 0xffff0000u);
+            w[4] = __uint_as_float(packed.z << 16), w[5] = __uint_as_float(packed.z & 0xffff0000u);
+            w[6] = __uint_as_float(packed.w << 16), w[7] = __uint_as_float(packed.w & 0xffff0000u);
+#pragma unroll
+            for (int i = 0; i < FEW_ROWS_M; ++i) {
+                const float4 lo = *(const float4*)(a_row + i * K + k);
+                const float4 hi = *(const float4*)(a_row + i * K + k + 4);
+                float s = acc[i];
+                s = fmaf(lo.x, w[0], s), s = fmaf(lo.y, w[1], s), s = fmaf(lo.z, w[2], s), s = fmaf(lo.w, w[3], s);
+                s = fmaf(hi.x, w[4], s), s = fmaf(hi.y, w[5], s), s = fmaf(hi.z, w[6], s), s = fmaf(hi.w, w[7], s);
+                acc[i] = s;
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < FEW_ROWS_M; ++i) {
+        float s = acc[i];
+        s += __shfl_xor(s, 1, HB_WAVE);
+        s += __shfl_xor(s, 2, HB_WAVE);
+        if (part == 0 && n < N && i < rows) C[(size_t)(m0 + i) * ldc + n] = s;
+    }
+}
+
+static bool few_rows_takes(const void* A, int a_dtype, const void* W, int w_dtype, int c_dtype, int M, int K, int lda,
+                           int ldw, int accumulate) {
+    return a_dtype == 0 && w_dtype == 1 && c_dtype == 0 && !accumulate && M <= 32 && K % 32 == 0 && K <= FEW_ROWS_K && lda % 4 == 0 &&
+           ldw % 8 == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0;
+}
+
 // C[M, N] (+)= A[M, K] * W[N, K]^T with row strides lda, ldw, ldc (in elements).
 extern "C" int hb_gemm_plain(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype,
                              int M, int N, int K, int lda, int ldw, int ldc, int accumulate,
@@ -116,6 +183,21 @@ extern "C" int hb_gemm_plain(const void* A, int a_dtype, const void* W, int w_dt
     }
     HB_CHECK_LAUNCH("gemm_plain");
     return 0;
+}
+
+// The same product for callers whose k is short (a narrow middle): few rows take the kernel made for them.
+extern "C" int hb_gemm_plain_short_k(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype,
+                                     int M, int N, int K, int lda, int ldw, int ldc, int accumulate,
+                                     hipStream_t stream) {
+    HB_REQUIRE(M > 0 && N > 0 && K > 0, "gemm: empty problem (M=%d, N=%d, K=%d)", M, N, K);
+    HB_REQUIRE(lda >= K && ldw >= K && ldc >= N, "gemm: a row stride is smaller than its row");
+    if (few_rows_takes(A, a_dtype, W, w_dtype, c_dtype, M, K, lda, ldw, accumulate)) {
+        gemm_few_rows_kernel<<<dim3((N + 15) / 16, (M + FEW_ROWS_M - 1) / FEW_ROWS_M), HB_WAVE, 0, stream>>>(
+            (const float*)A, (const bf16*)W, (float*)C, M, N, K, lda, ldw, ldc);
+        HB_CHECK_LAUNCH("gemm_few_rows");
+        return 0;
+    }
+    return hb_gemm_plain(A, a_dtype, W, w_dtype, C, c_dtype, M, N, K, lda, ldw, ldc, accumulate, stream);
 }
 
 // A batch of such products in one launch: product b reads A + b * batch_a, W + b * batch_w and writes

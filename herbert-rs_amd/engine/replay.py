@@ -26,7 +26,7 @@ from .batch import StepEntry
 from .engine import Engine
 
 
-PARTIAL_PAGES = 64
+PARTIAL_PAGES = 256
 
 
 class Replayer:

@@ -448,7 +448,8 @@ def relu_squared(z, out):
 
 def gemm_plain_columns(a, col0, K, w, c, accumulate=False):
     """c[M, N] (+)= a[:, col0:col0 + K] @ w[N, K]^T in float32 arithmetic: the product of some columns of
-    wider rows, read where they lie."""
+    wider rows, read where they lie. (Up to 32 float32 rows times bfloat16 rows, k in steps of 32: a kernel of
+    more and smaller workgroups than the tiled one, which a short k leaves with few.)"""
     _check(a, "a", None, (None, None))
     _check(w, "w", None, (None, K))
     M, lda = a.shape
@@ -458,5 +459,5 @@ def gemm_plain_columns(a, col0, K, w, c, accumulate=False):
     _check(c, "c", None, (M, N))
     if accumulate and c.dtype != torch.float32:
         raise BackendError("gemm: accumulation needs a float32 output")
-    lib.call("gemm_plain", "hb_gemm_plain", a.data_ptr() + col0 * a.element_size(), dtype_code(a), w.data_ptr(),
+    lib.call("gemm_plain", "hb_gemm_plain_short_k", a.data_ptr() + col0 * a.element_size(), dtype_code(a), w.data_ptr(),
              dtype_code(w), c.data_ptr(), dtype_code(c), M, N, K, lda, K, N, 1 if accumulate else 0, _stream())

@@ -361,3 +361,18 @@ def test_experts_products_and_the_shared_experts_gated_sum():
             moe.gemm_plain(act, down_w, out, routing, gather=False)
         moe.combine(out, routing, x, shared=shared.to(DEV), gate=(rows.to(DEV).contiguous(), E))
         assert torch.allclose(x.cpu(), want, atol=tol, rtol=tol), f"{dtype}"
+
+
+# ---------------------------------------------------------------- the second product of a pair through a narrow middle
+@pytest.mark.parametrize("M,N,K,col0,ld", [(1, 128, 32, 0, 32), (8, 2048, 128, 260, 400), (32, 48, 64, 4, 72), (7, 50, 96, 8, 104),
+                                           (33, 64, 32, 0, 32), (5, 40, 24, 0, 24), (6, 32, 32, 3, 40)])
+def test_product_of_some_columns_with_a_short_k(M, N, K, col0, ld):
+    """Few rows of bfloat16 weights take a kernel of their own (k in steps of 32, rows on 16-byte borders);
+    more rows, another k or columns off those borders take the tiled one: both against the plain product."""
+    a, w = rand(M, ld, seed=M), rand(N, K, seed=N, scale=0.3)
+    for dtype, tol in ((torch.bfloat16, 2e-5), (torch.float32, 2e-5)):
+        wd = w.to(dtype)
+        c = torch.full((M, N), 9.0, device=DEV)
+        ops.gemm_plain_columns(a.to(DEV), col0, K, wd.to(DEV), c)
+        want = a[:, col0:col0 + K].double() @ wd.double().T
+        assert torch.allclose(c.cpu().double(), want, atol=tol, rtol=tol), dtype
