@@ -37,10 +37,13 @@ class AttentionMixerConfig:
 
     @staticmethod
     def from_reader(r, where):
-        t = _section(r.raw, "q_temp", where + ".")
+        # (a mixer without "q_temp", or with null there, has queries that do not grow: coef 0)
+        coef, every = 0.0, 1
+        if r.raw.get("q_temp") is not None:
+            t = _section(r.raw, "q_temp", where + ".")
+            coef, every = t.number("coef", required=True), t.integer("every", required=True)
         c = AttentionMixerConfig(*(r.integer(k, required=True) for k in ("heads", "kv_heads", "dim", "vdim")),
-                                 r.number("scale", required=True), t.number("coef", required=True),
-                                 t.integer("every", required=True))
+                                 r.number("scale", required=True), coef, every)
         if min(c.heads, c.kv_heads, c.dim, c.vdim, c.q_temp_every) <= 0 or c.heads % c.kv_heads:
             raise ConfigError(f"config.json: {where}: sizes must be positive and heads a multiple of kv_heads")
         return c
@@ -96,12 +99,14 @@ class ExpertsConfig:
     groups: int
     keep: int
     ff: int
-    shared_ff: int
+    shared_ff: Optional[int]         # None: no shared expert
 
     def to_dict(self):
-        return {"kind": "moe", "expert": {"ff": self.ff},
-                "router": {"experts": self.experts, "top": self.top, "groups": {"count": self.groups, "keep": self.keep}},
-                "shared": {"ff": self.shared_ff}}
+        d = {"kind": "moe", "expert": {"ff": self.ff},
+             "router": {"experts": self.experts, "top": self.top, "groups": {"count": self.groups, "keep": self.keep}}}
+        if self.shared_ff is not None:
+            d["shared"] = {"ff": self.shared_ff}
+        return d
 
 
 def _mlp(r, where):
@@ -114,12 +119,16 @@ def _mlp(r, where):
     if kind != "moe":
         raise ConfigError(f"config.json: {where}: unknown feed-forward kind {kind!r} (known: 'dense', 'moe')")
     expert, router = _section(r.raw, "expert", where + "."), _section(r.raw, "router", where + ".")
-    groups = _section(router.raw, "groups", where + ".router.")
-    shared = _section(r.raw, "shared", where + ".")
-    c = ExpertsConfig(router.integer("experts", required=True), router.integer("top", required=True),
-                      groups.integer("count", required=True), groups.integer("keep", required=True),
-                      expert.integer("ff", required=True), shared.integer("ff", required=True))
-    if not 0 < c.top <= c.experts or c.ff <= 0 or c.shared_ff <= 0:
+    # (a router without "groups" has one group of all experts; a feed-forward without "shared" no shared expert)
+    count, keep, shared_ff = 1, 1, None
+    if router.raw.get("groups") is not None:
+        groups = _section(router.raw, "groups", where + ".router.")
+        count, keep = groups.integer("count", required=True), groups.integer("keep", required=True)
+    if r.raw.get("shared") is not None:
+        shared_ff = _section(r.raw, "shared", where + ".").integer("ff", required=True)
+    c = ExpertsConfig(router.integer("experts", required=True), router.integer("top", required=True), count, keep,
+                      expert.integer("ff", required=True), shared_ff)
+    if not 0 < c.top <= c.experts or c.ff <= 0 or (c.shared_ff is not None and c.shared_ff <= 0):
         raise ConfigError(f"config.json: {where}: top must be within 1..experts and the widths positive")
     if c.groups <= 0 or c.experts % c.groups or not 0 < c.keep <= c.groups or c.top > c.keep * (c.experts // c.groups):
         raise ConfigError(f"config.json: {where}: {c.top} experts cannot come from {c.keep} of {c.groups} equal "

@@ -41,8 +41,9 @@ def _feed_forward(cfg, m, p):
                                          "names": {"up": p + "up", "down": p + "down"}})
     names = {"router": p + "router", "router_bias": p + "correction", "gate": p + "e{e}.gate", "up": p + "e{e}.up",
              "down": p + "e{e}.down"}
-    shared = {"intermediate_size": m.shared_ff,
-              "names": {k: p + "shared." + k for k in ("gate", "up", "down", "sg")}}
+    shared = None
+    if m.shared_ff is not None:
+        shared = {"intermediate_size": m.shared_ff, "names": {k: p + "shared." + k for k in ("gate", "up", "down", "sg")}}
     return PartSpec("routed_experts", {"hidden_size": cfg.hidden_size, "intermediate_size": m.ff,
                                        "experts": m.experts, "top": m.top, "names": names, "routing": "scores",
                                        "groups": m.groups, "keep": m.keep, "activation": "silu",

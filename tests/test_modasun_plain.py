@@ -213,3 +213,20 @@ def test_configuration_errors():
             arch.config_class.from_dict(raw)
     with pytest.raises(ConfigError):
         resolve_architecture({"architecture": "Modasum"})
+
+
+def test_sections_that_a_configuration_may_leave_out():
+    """No "q_temp": queries that do not grow; no "groups": one group of all experts; no "shared": no shared expert."""
+    raw = json.loads(json.dumps(CONFIGS["P"][0]))
+    del raw["layers"][1]["mixer"]["q_temp"]
+    del raw["layers"][2]["mixer"]["q_temp"]
+    del raw["layers"][0]["mlp"]["router"]["groups"]
+    del raw["layers"][0]["mlp"]["shared"]
+    del raw["layers"][3]["mlp"]["router"]["groups"]
+    del raw["layers"][3]["mlp"]["shared"]
+    arch = resolve_architecture(raw)
+    cfg = arch.config_class.from_dict(raw)
+    assert cfg.layers[1].mixer.q_temp_coef == 0.0 and cfg.layers[0].mlp.groups == cfg.layers[0].mlp.keep == 1
+    assert cfg.layers[0].mlp.shared_ff is None
+    needs = Model(arch.build_spec(cfg)).tensor_needs()
+    assert "l0.mlp.router" in needs and not any(k.startswith("l0.mlp.shared") for k in needs)
