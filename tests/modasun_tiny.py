@@ -85,7 +85,19 @@ def _s():
     layers = [with_mlp(attention(2, 1, 160, 144, 0.08, 0.3, 1), moe(12, 4, 1, 1, 80, 48)),
               with_mlp(delta(4, 2, 40, 48, 3, 12, 20), moe(12, 4, 1, 1, 80, 48))]
     layers += [again(layers, 1), with_mlp(attention(6, 3, 32, 16, 0.2, 0.1, 50), dense(96))]
-    return model(320, 192, layers, eps=2e-5, alpha=2.5, embed_scale=9.0)
+    return model(320, 192, layers, eps=2e-5, alpha=2.25, embed_scale=9.0)
+
+
+def _n():
+    # N: the sections that a configuration may leave out: an attention whose queries do not grow, routers
+    #    without groups, feed-forwards without a shared expert (one of the two routed layers keeps its own)
+    bare = {"kind": "moe", "expert": {"ff": 48}, "router": {"experts": 5, "top": 2}}
+    plain_attention = {"type": "attention", "mixer": {"heads": 3, "kv_heads": 3, "dim": 32, "vdim": 48, "scale": 0.25}}
+    grouped = {"kind": "moe", "expert": {"ff": 32}, "router": {"experts": 6, "top": 2, "groups": {"count": 2, "keep": 1}}}
+    layers = [with_mlp(plain_attention, bare), with_mlp(delta(2, 2, 32, 48, 3, 8, 8), grouped),
+              with_mlp(attention(3, 1, 32, 48, 0.2, 0.4, 8), dict(bare, shared={"ff": 40}))]
+    layers.append(again(layers, 0))
+    return model(160, 96, layers, eps=4e-6, alpha=1.3, embed_scale=4.0)
 
 
 def _w():
@@ -104,7 +116,7 @@ def _f():
     return model(384, 128, layers, eps=1e-6, alpha=1.5, embed_scale=2.0)
 
 
-CONFIGS = {"F": (_f(), 26, 0.09), "P": (_p(), 21, 0.12), "Q": (_q(), 22, 0.09), "R": (_r(), 23, 0.15), "S": (_s(), 24, 0.08), "W": (_w(), 25, 0.05)}
+CONFIGS = {"F": (_f(), 26, 0.09), "P": (_p(), 21, 0.12), "Q": (_q(), 22, 0.09), "R": (_r(), 23, 0.15), "S": (_s(), 24, 0.08), "N": (_n(), 27, 0.1), "W": (_w(), 25, 0.05)}
 
 
 def make_folder(root, name, dtype="float32", scale=None, set_to=None, tag=""):

@@ -71,14 +71,16 @@ def softmax_attention(q, k, v, scale):
 
 
 def attention_mixer(h, w, m, eps):
-    """h [T, W]; w: q, k, v, o; m: heads, kv_heads, dim, vdim, scale, q_temp {coef, every}."""
+    """h [T, W]; w: q, k, v, o; m: heads, kv_heads, dim, vdim, scale, q_temp {coef, every} (or none: the
+    queries stay as they are)."""
     T = h.shape[0]
     H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     q = rms_scale(linear(h, w["q"]).view(T, H, D), eps)
     k = rms_scale(linear(h, w["k"]).view(T, G, D), eps)
     v = linear(h, w["v"]).view(T, G, V)
-    temp = query_temperature(torch.arange(T), m["q_temp"]["coef"], m["q_temp"]["every"]).to(h.dtype)
-    q = q * temp[:, None, None]
+    if m.get("q_temp") is not None:
+        temp = query_temperature(torch.arange(T), m["q_temp"]["coef"], m["q_temp"]["every"]).to(h.dtype)
+        q = q * temp[:, None, None]
     heads = []
     for head in range(H):
         g = head // (H // G)
@@ -168,10 +170,11 @@ def choose_experts(scores, correction, top, groups, keep):
 
 
 def moe_ff(h, w, m):
-    """w: router, correction, e<i>.gate/up/down, shared.gate/up/down/sg; m: the layer's 'mlp' entry."""
+    """w: router, correction, e<i>.gate/up/down, shared.gate/up/down/sg; m: the layer's 'mlp' entry (without
+    'groups': one group of all experts; without 'shared': no shared expert)."""
     r = m["router"]
     E, top = r["experts"], r["top"]
-    groups, keep = r["groups"]["count"], r["groups"]["keep"]
+    groups, keep = (r["groups"]["count"], r["groups"]["keep"]) if r.get("groups") is not None else (1, 1)
     scores = sigmoid(linear(h, w["router"]))
     out = torch.zeros(h.shape[0], w["e0.down"].shape[0], dtype=h.dtype)
     for t in range(h.shape[0]):
@@ -179,6 +182,8 @@ def moe_ff(h, w, m):
         total = sum(scores[t, e] for e in chosen) + 1e-20
         for e in chosen:
             out[t] += scores[t, e] / total * glu_expert(h[t], w[f"e{e}.gate"], w[f"e{e}.up"], w[f"e{e}.down"])
+    if m.get("shared") is None:
+        return out
     shared = glu_expert(h, w["shared.gate"], w["shared.up"], w["shared.down"])
     return out + sigmoid(linear(h, w["shared.sg"])) * shared
 

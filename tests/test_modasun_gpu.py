@@ -65,7 +65,7 @@ def feed(engine, slot, tokens, cuts):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["P", "Q", "R", "S"])
+@pytest.mark.parametrize("name", ["P", "Q", "R", "S", "N"])
 def test_whole_prompts_and_token_by_token(name, dtype, model_root):
     folder = make_folder(model_root, name, dtype)
     vocab = CONFIGS[name][0]["vocab"]
@@ -99,7 +99,7 @@ def test_portions_of_several_sizes_and_slots_used_again(name, dtype, model_root)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["P", "Q", "R", "S"])
+@pytest.mark.parametrize("name", ["P", "Q", "R", "S", "N"])
 def test_unequal_batches_against_each_alone(name, dtype, model_root):
     folder = make_folder(model_root, name, dtype)
     vocab = CONFIGS[name][0]["vocab"]

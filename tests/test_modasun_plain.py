@@ -114,7 +114,7 @@ def test_the_choice_of_experts():
 
 def test_mixture_of_experts_weights_and_the_shared_expert():
     W, F, Fs, E, T = 8, 6, 5, 4, 7
-    m = {"router": {"experts": E, "top": 2, "groups": {"count": 2, "keep": 2}}}
+    m = {"router": {"experts": E, "top": 2, "groups": {"count": 2, "keep": 2}}, "shared": {"ff": Fs}}
     w = {"router": rand(E, W, seed=1), "correction": 0.1 * rand(E, seed=2), "shared.gate": rand(Fs, W, seed=3),
          "shared.up": rand(Fs, W, seed=4), "shared.down": rand(W, Fs, seed=5), "shared.sg": rand(1, W, seed=6)}
     for e in range(E):
@@ -130,6 +130,8 @@ def test_mixture_of_experts_weights_and_the_shared_expert():
             y = torch.nn.functional.silu(h[t] @ w[f"e{e}.gate"].T) * (h[t] @ w[f"e{e}.up"].T)
             want[t] += s[t, e] / (s[t, e] + s[t, other]) * (y @ w[f"e{e}.down"].T)
     shared = (torch.nn.functional.silu(h @ w["shared.gate"].T) * (h @ w["shared.up"].T)) @ w["shared.down"].T
+    bare = plain.moe_ff(h, w, {"router": {"experts": E, "top": 2}})       # one group, no shared expert
+    assert torch.allclose(bare, want, atol=1e-10)
     want += torch.sigmoid(h @ w["shared.sg"].T) * shared
     assert torch.allclose(got, want, atol=1e-10)
     x = rand(4, W, seed=8)
@@ -142,7 +144,9 @@ def test_configuration_spec_and_needs(name):
     raw = CONFIGS[name][0]
     arch = resolve_architecture(raw)
     cfg = arch.config_class.from_dict(raw)
-    assert arch.name == "Modasun" and cfg.to_dict() == raw
+    assert arch.name == "Modasun" and arch.config_class.from_dict(cfg.to_dict()).to_dict() == cfg.to_dict()
+    if name != "N":                      # (N leaves sections out, which are written back with what they default to)
+        assert cfg.to_dict() == raw
     model = Model(arch.build_spec(cfg))
     needs = model.tensor_needs()
     W = raw["width"]
@@ -175,7 +179,10 @@ def test_configuration_spec_and_needs(name):
             E = mlp["router"]["experts"]
             assert needs[p + "mlp.router"].shape == (E, W) and needs[p + "mlp.correction"].shape == (E,)
             assert needs[p + f"mlp.e{E - 1}.down"].shape == (W, mlp["expert"]["ff"]) and p + f"mlp.e{E}.down" not in needs
-            assert needs[p + "mlp.shared.up"].shape == (mlp["shared"]["ff"], W) and needs[p + "mlp.shared.sg"].shape == (1, W)
+            if "shared" in mlp:
+                assert needs[p + "mlp.shared.up"].shape == (mlp["shared"]["ff"], W) and needs[p + "mlp.shared.sg"].shape == (1, W)
+            else:
+                assert not any(k.startswith(p + "mlp.shared") for k in needs)
         elif mlp is not None:
             assert needs[p + "mlp.up"].shape == (mlp["ff"], W) and needs[p + "mlp.down"].shape == (W, mlp["ff"])
 
