@@ -16,10 +16,26 @@ HB_MODULE_ERROR_SLOT()
 #define TILE_N 64
 #define TILE_K 16
 
+// What a product may do to a sum before it stores it: nothing (rate null), or turn the pre-activation of a
+// decay into the decay itself, exp(-exp(rate[n / D]) * softplus(sum + bias[n])) for column n (float32; the
+// arithmetic of hb_channel_decay, which does the same to rows that lie in memory).
+struct DecayEpilogue {
+    const float* rate;
+    const float* bias;
+    int D;
+};
+
+__device__ __forceinline__ float decay_of(const DecayEpilogue& ep, float sum, int n) {
+    const float a = sum + ep.bias[n];
+    const float softplus = a > 20.f ? a : log1pf(expf(a));
+    return expf(-expf(ep.rate[n / ep.D]) * softplus);
+}
+
 template <class TA, class TW, class TC, bool ACCUM>
 __global__ void __launch_bounds__(256)
 gemm_plain_kernel(const TA* __restrict__ A, const TW* __restrict__ W, TC* __restrict__ C, int M, int N,
-                  int K, int lda, int ldw, int ldc, size_t batch_a, size_t batch_w, size_t batch_c) {
+                  int K, int lda, int ldw, int ldc, size_t batch_a, size_t batch_w, size_t batch_c,
+                  DecayEpilogue ep) {
     // (blockIdx.z: one of a batch of products whose operands lie batch_* elements apart)
     A += blockIdx.z * batch_a;
     W += blockIdx.z * batch_w;
@@ -79,7 +95,7 @@ gemm_plain_kernel(const TA* __restrict__ A, const TW* __restrict__ W, TC* __rest
             if (ACCUM)
                 C[idx] = hb_from_float<TC>(hb_to_float(C[idx]) + acc[i][j]);
             else
-                C[idx] = hb_from_float<TC>(acc[i][j]);
+                C[idx] = hb_from_float<TC>(ep.rate ? decay_of(ep, acc[i][j], n) : acc[i][j]);
         }
     }
 }
@@ -87,14 +103,14 @@ gemm_plain_kernel(const TA* __restrict__ A, const TW* __restrict__ W, TC* __rest
 template <class TA, class TW, class TC>
 static void launch(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldw, int ldc,
                    int accumulate, hipStream_t stream, int batch = 1, size_t batch_a = 0, size_t batch_w = 0,
-                   size_t batch_c = 0) {
+                   size_t batch_c = 0, DecayEpilogue ep = DecayEpilogue{nullptr, nullptr, 1}) {
     dim3 grid((N + TILE_N - 1) / TILE_N, (M + TILE_M - 1) / TILE_M, batch);
     if (accumulate)
         gemm_plain_kernel<TA, TW, TC, true><<<grid, 256, 0, stream>>>(
-            (const TA*)A, (const TW*)W, (TC*)C, M, N, K, lda, ldw, ldc, batch_a, batch_w, batch_c);
+            (const TA*)A, (const TW*)W, (TC*)C, M, N, K, lda, ldw, ldc, batch_a, batch_w, batch_c, ep);
     else
         gemm_plain_kernel<TA, TW, TC, false><<<grid, 256, 0, stream>>>(
-            (const TA*)A, (const TW*)W, (TC*)C, M, N, K, lda, ldw, ldc, batch_a, batch_w, batch_c);
+            (const TA*)A, (const TW*)W, (TC*)C, M, N, K, lda, ldw, ldc, batch_a, batch_w, batch_c, ep);
 }
 
 
@@ -108,7 +124,7 @@ static void launch(const void* A, const void* W, void* C, int M, int N, int K, i
 #define FEW_ROWS_K 1024
 __global__ void __launch_bounds__(HB_WAVE)
 gemm_few_rows_kernel(const float* __restrict__ A, const bf16* __restrict__ W, float* __restrict__ C, int M, int N,
-                     int K, int lda, int ldw, int ldc) {
+                     int K, int lda, int ldw, int ldc, DecayEpilogue ep) {
     __shared__ __attribute__((aligned(16))) float rows_of_a[FEW_ROWS_M * FEW_ROWS_K];
     const int lane = threadIdx.x;
     const int n = blockIdx.x * 16 + lane / 4;
@@ -149,10 +165,16 @@ gemm_few_rows_kernel(const float* __restrict__ A, const bf16* __restrict__ W, fl
     }
 #pragma unroll
     for (int i = 0; i < FEW_ROWS_M; ++i) {
-        float s = acc[i];
-        s += __shfl_xor(s, 1, HB_WAVE);
-        s += __shfl_xor(s, 2, HB_WAVE);
-        if (part == 0 && n < N && i < rows) C[(size_t)(m0 + i) * ldc + n] = s;
+        acc[i] += __shfl_xor(acc[i], 1, HB_WAVE);
+        acc[i] += __shfl_xor(acc[i], 2, HB_WAVE);
+    }
+    // (all four lanes of a column hold its sums: each stores, and first turns into a decay, every fourth row)
+    static_assert(FEW_ROWS_M % 4 == 0, "the rows are dealt out to a column's four lanes");
+#pragma unroll
+    for (int j = 0; j < FEW_ROWS_M / 4; ++j) {
+        const float s = part == 0 ? acc[4 * j] : part == 1 ? acc[4 * j + 1] : part == 2 ? acc[4 * j + 2] : acc[4 * j + 3];
+        const int i = 4 * j + part;
+        if (n < N && i < rows) C[(size_t)(m0 + i) * ldc + n] = ep.rate ? decay_of(ep, s, n) : s;
     }
 }
 
@@ -186,18 +208,34 @@ extern "C" int hb_gemm_plain(const void* A, int a_dtype, const void* W, int w_dt
 }
 
 // The same product for callers whose k is short (a narrow middle): few rows take the kernel made for them.
+// A_log [N / D] and dt_bias [N], both or neither: the sums are a decay's pre-activations, and what is stored is
+// the decay a column (float32 in and out, no accumulation).
 extern "C" int hb_gemm_plain_short_k(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype,
                                      int M, int N, int K, int lda, int ldw, int ldc, int accumulate,
-                                     hipStream_t stream) {
+                                     const float* A_log, const float* dt_bias, int D, hipStream_t stream) {
     HB_REQUIRE(M > 0 && N > 0 && K > 0, "gemm: empty problem (M=%d, N=%d, K=%d)", M, N, K);
     HB_REQUIRE(lda >= K && ldw >= K && ldc >= N, "gemm: a row stride is smaller than its row");
+    HB_REQUIRE((A_log == nullptr) == (dt_bias == nullptr), "gemm: a decay needs its rate and its bias");
+    HB_REQUIRE(!A_log || (D > 0 && N % D == 0 && c_dtype == 0 && !accumulate),
+               "gemm: a decay is float32, stored and not added, %d columns in heads of %d", N, D);
+    const DecayEpilogue ep{A_log, dt_bias, A_log ? D : 1};
     if (few_rows_takes(A, a_dtype, W, w_dtype, c_dtype, M, K, lda, ldw, accumulate)) {
         gemm_few_rows_kernel<<<dim3((N + 15) / 16, (M + FEW_ROWS_M - 1) / FEW_ROWS_M), HB_WAVE, 0, stream>>>(
-            (const float*)A, (const bf16*)W, (float*)C, M, N, K, lda, ldw, ldc);
+            (const float*)A, (const bf16*)W, (float*)C, M, N, K, lda, ldw, ldc, ep);
         HB_CHECK_LAUNCH("gemm_few_rows");
         return 0;
     }
-    return hb_gemm_plain(A, a_dtype, W, w_dtype, C, c_dtype, M, N, K, lda, ldw, ldc, accumulate, stream);
+    if (!A_log) return hb_gemm_plain(A, a_dtype, W, w_dtype, C, c_dtype, M, N, K, lda, ldw, ldc, accumulate, stream);
+    HB_REQUIRE((M + TILE_M - 1) / TILE_M <= 65535, "gemm: M=%d exceeds the grid", M);
+    switch (a_dtype * 2 + w_dtype) {
+        case 0: launch<float, float, float>(A, W, C, M, N, K, lda, ldw, ldc, 0, stream, 1, 0, 0, 0, ep); break;
+        case 1: launch<float, bf16, float>(A, W, C, M, N, K, lda, ldw, ldc, 0, stream, 1, 0, 0, 0, ep); break;
+        case 2: launch<bf16, float, float>(A, W, C, M, N, K, lda, ldw, ldc, 0, stream, 1, 0, 0, 0, ep); break;
+        case 3: launch<bf16, bf16, float>(A, W, C, M, N, K, lda, ldw, ldc, 0, stream, 1, 0, 0, 0, ep); break;
+        default: HB_REQUIRE(false, "gemm: unknown dtypes (%d, %d)", a_dtype, w_dtype);
+    }
+    HB_CHECK_LAUNCH("gemm_plain");
+    return 0;
 }
 
 // A batch of such products in one launch: product b reads A + b * batch_a, W + b * batch_w and writes

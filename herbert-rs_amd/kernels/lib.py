@@ -33,7 +33,7 @@ SIGNATURES = {
     },
     "gemm_plain": {
         "hb_gemm_plain": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P],
-        "hb_gemm_plain_short_k": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P],
+        "hb_gemm_plain_short_k": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _I, _P],
         "hb_gemm_plain_batched": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _SZ, _SZ, _SZ, _P],
     },
     "recurrent": {

@@ -446,10 +446,13 @@ def relu_squared(z, out):
     lib.call("elementwise", "hb_relu_squared", z.data_ptr(), out.data_ptr(), dtype_code(out), z.numel(), _stream())
 
 
-def gemm_plain_columns(a, col0, K, w, c, accumulate=False):
+def gemm_plain_columns(a, col0, K, w, c, accumulate=False, decay=None):
     """c[M, N] (+)= a[:, col0:col0 + K] @ w[N, K]^T in float32 arithmetic: the product of some columns of
     wider rows, read where they lie. (Up to 32 float32 rows times bfloat16 rows, k in steps of 32: a kernel of
-    more and smaller workgroups than the tiled one, which a short k leaves with few.)"""
+    more and smaller workgroups than the tiled one, which a short k leaves with few.)
+    decay (a_log f32 [N / D], dt_bias f32 [N], D): the sums are a decay's pre-activations, and c (float32, not
+    added to) takes the decays themselves, exp(-exp(a_log[n // D]) softplus(sum + dt_bias[n])), as
+    `recurrent.channel_decay` makes them from rows in memory."""
     _check(a, "a", None, (None, None))
     _check(w, "w", None, (None, K))
     M, lda = a.shape
@@ -459,5 +462,14 @@ def gemm_plain_columns(a, col0, K, w, c, accumulate=False):
     _check(c, "c", None, (M, N))
     if accumulate and c.dtype != torch.float32:
         raise BackendError("gemm: accumulation needs a float32 output")
+    a_log = dt_bias = D = 0
+    if decay is not None:
+        rate, bias, D = decay
+        if accumulate or c.dtype != torch.float32 or D <= 0 or N % D:
+            raise BackendError("gemm: a decay is float32, stored and not added to, its columns whole heads")
+        _check(rate, "A_log", torch.float32, (N // D,))
+        _check(bias, "dt_bias", torch.float32, (N,))
+        a_log, dt_bias = rate.data_ptr(), bias.data_ptr()
     lib.call("gemm_plain", "hb_gemm_plain_short_k", a.data_ptr() + col0 * a.element_size(), dtype_code(a), w.data_ptr(),
-             dtype_code(w), c.data_ptr(), dtype_code(c), M, N, K, lda, K, N, 1 if accumulate else 0, _stream())
+             dtype_code(w), c.data_ptr(), dtype_code(c), M, N, K, lda, K, N, 1 if accumulate else 0, a_log, dt_bias,
+             int(D), _stream())

@@ -154,10 +154,14 @@ class GatedDelta(Part):
             gate_rows, gate_off = rt.buffer("delta_gate", (T, self.heads * self.vdim), torch.float32), 0
             ops.gemm_plain_columns(proj, self.g_off, self.g_width, self.g2, gate_rows)
             decay_rows, decay_off = rt.buffer("delta_decay", (T, self.decay_width), torch.float32), 0
-            ops.gemm_plain_columns(proj, self.a_off, self.a_width, self.a2, decay_rows)
+            # (a decay a channel leaves this product as the decay itself: softplus and exponentials where the sum is stored)
+            ops.gemm_plain_columns(proj, self.a_off, self.a_width, self.a2, decay_rows,
+                                   decay=(self.a_log, self.dt_bias, self.dim) if self.decay == "channel" else None)
         if self.decay == "channel":
-            factors = rt.buffer("delta_decay", (T, self.decay_width), torch.float32)
-            recurrent.channel_decay(decay_rows, decay_off, self.a_log, self.dt_bias, factors, self.heads, self.dim)
+            factors = decay_rows
+            if self.low_rank is None:
+                factors = rt.buffer("delta_decay", (T, self.decay_width), torch.float32)
+                recurrent.channel_decay(decay_rows, decay_off, self.a_log, self.dt_bias, factors, self.heads, self.dim)
             recurrent.gated_delta(qkv, proj, self.b_off, 0, None, None, state, ctx.meta, o,
                                   self.kv_heads, self.heads, self.dim, self.vdim, decay=factors)
         else:

@@ -376,3 +376,13 @@ def test_product_of_some_columns_with_a_short_k(M, N, K, col0, ld):
         ops.gemm_plain_columns(a.to(DEV), col0, K, wd.to(DEV), c)
         want = a[:, col0:col0 + K].double() @ wd.double().T
         assert torch.allclose(c.cpu().double(), want, atol=tol, rtol=tol), dtype
+        # the same product leaving the decays of which its sums are the pre-activations, for every size of a head
+        # that divides the columns: exp(-exp(A_log[head]) softplus(sum + dt_bias[column]))
+        for D in {1, 8, N // 2, N}:
+            if N % D:
+                continue
+            rate, bias = rand(N // D, seed=D + 1), rand(N, seed=D + 2, scale=2.0)
+            g = torch.full((M, N), 9.0, device=DEV)
+            ops.gemm_plain_columns(a.to(DEV), col0, K, wd.to(DEV), g, decay=(rate.to(DEV), bias.to(DEV), D))
+            want_g = torch.exp(-torch.exp(rate.double()).repeat_interleave(D) * plain.softplus(want + bias.double()))
+            assert torch.allclose(g.cpu().double(), want_g, atol=tol, rtol=tol), (dtype, D)
