@@ -68,8 +68,8 @@ moe_route_kernel(const float* __restrict__ logits, int ld, const float* __restri
 }
 
 // Routing by scores s = sigmoid(logit). The choice runs on s + correction, the weights on s itself:
-// the experts form n_groups equal groups of neighbours, a group is worth the sum of its two largest
-// choice scores, only the experts of the `keep` best groups can be chosen (the lower index of equals,
+// the experts form n_groups equal runs of adjacent experts, a group is worth the two highest of its
+// selection values, added; only the experts of the `keep` best groups can be chosen (the lower index of equals,
 // for groups as for experts), and the chosen experts' scores are divided by their sum + 1e-20.
 // One wave a token; the scores lie in LDS.
 __global__ void __launch_bounds__(HB_WAVE)

@@ -44,7 +44,7 @@ def route(logits, bias, routing, scores=False, groups=1, keep=1):
     """logits f32 [T, E] (+ bias f32 [E]) -> routing (see Routing): the largest logits + bias, weighed by a
     softmax over the chosen. The logits' rows may be wider than E (their first E columns count).
     scores=True: s = sigmoid(logit), the choice runs on s + bias within the `keep` best of `groups` equal
-    groups of neighbours (a group is worth its two largest choice scores), and the weights are the chosen
+    runs of adjacent experts (a group is worth its top two selection values), and the weights are the chosen
     experts' s over their sum."""
     r = routing
     _check(logits, "logits", torch.float32, (r.T, None))

@@ -1,7 +1,7 @@
 """Modasun as data: which parts each layer has and what its tensors are called.
 
 A layer is the "postnorm" arrangement: x <- norm1(alpha x + mixer(x)), x <- norm2(alpha x + ff(x)), the norms
-RMS norms whose weights are stored around zero. The mixer is a softmax attention without a rotation
+RMS norms whose stored weights are offsets from one. The mixer is a softmax attention without a rotation
 ("attention": queries and keys divided by their root mean square a head, a query growing with the logarithm
 of its position, values of a size of their own) or a gated delta rule with a decay a key channel
 ("channel_delta": two-step projections for the decay and the sigmoid gate); the feed-forward is dense

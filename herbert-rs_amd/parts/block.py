@@ -4,7 +4,7 @@
 and their sum joins the residual stream times a constant.
 
 "postnorm": x <- norm_post_mixer(alpha x + mixer(x)); x <- norm_post_ff(alpha x + feed_forward(x)): the parts
-read x itself, and each norm comes after its sum.
+take x as it is, and each norm comes after its sum.
 
 "prenorm": x += mixer(norm_input(x)); x += feed_forward(norm_post_mixer(x)), the
 arrangement of the reference's two-norm layer
@@ -126,7 +126,7 @@ class ParallelBlock(Part):
 @register("block", "postnorm")
 class PostNormBlock(Part):
     """x <- norm_post_mixer(alpha x + mixer(x)), then x <- norm_post_ff(alpha x + feed_forward(x)) (the second
-    step only where the layer has a feed-forward). The parts read x itself, in the compute dtype, and add
+    step only where the layer has a feed-forward). The parts take x as it is, in the compute dtype, and add
     their outputs, as they always do, to float32 rows: rows that already hold alpha x. One kernel between
     two parts norms those rows into x, writes the copy that the next part reads and alpha x where it adds;
     the one after a layer's last part does so for the next layer too, if that is such a block."""
@@ -158,7 +158,7 @@ class PostNormBlock(Part):
         rt = ctx.rt
         shape = tuple(x.shape)
         acc = rt.buffer("postnorm_sum", shape, torch.float32)
-        y = None if rt.exact else rt.buffer("postnorm_rows", shape)       # (float32: the parts read x itself)
+        y = None if rt.exact else rt.buffer("postnorm_rows", shape)       # (float32: the parts take x as it is)
         pending, ctx.pending_post = ctx.pending_post, None
         if pending != (x.data_ptr(), self.alpha):
             ops.postnorm(x, None, None, y, 0.0, self.alpha, acc=acc)

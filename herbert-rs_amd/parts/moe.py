@@ -9,7 +9,7 @@ fixed length, so a step's grid depends on its size only.
 
 Variants, each a parameter. `routing="scores"`: s = sigmoid(z); the choice runs on s + correction (a stored
 vector) and only within the `keep` best of `groups` equal groups of neighbouring experts, a group being worth
-the sum of its two largest choice scores; the weights are the chosen experts' s over their sum (+ 1e-20).
+the two highest of its selection values, added; the weights are the chosen experts' s over their sum (+ 1e-20).
 `activation="silu"`: an expert is W_down (silu(W_gate y) (W_up y)), nothing clamped. `shared_expert`: one more
 expert of that form and a width of its own that every token takes, its output times sigmoid(w_sg . y) (one
 number a token) added to the routed experts' sum.

@@ -1,6 +1,6 @@
 """Norms of the residual stream. RMSNorm as the reference computes it (crates/backends/backend_common/src/kernels.rs:54-64):
 y = x / sqrt(mean(x^2) + eps) * w, the weight used as stored (not 1 + w). A family whose weights are
-stored around zero gives `offset` 1: the kernels then see offset + w."""
+stored as an offset from one gives `offset` 1: the kernels then see offset + w."""
 from ..kernels import ops
 from ..weights import TensorNeed
 from .base import Part
@@ -19,7 +19,7 @@ class RMSNorm(Part):
     hands_on = True      # y = x * w / rms(x): a product may apply the 1 / rms to its sums instead (NormedRows)
 
     def __init__(self, size, eps, weight, offset=0.0):
-        """offset: added to the stored weight (1 for weights stored around zero)."""
+        """offset: added to the stored weight (1 for weights stored as offsets from one)."""
         self.size = int(size)
         self.eps = float(eps)
         self.weight_name = weight

@@ -27,7 +27,7 @@ def rms_scale(x, eps):
 
 
 def offset_norm(x, w, eps):
-    """The design's norm: the weight is stored around zero."""
+    """The design's norm: the stored weight is an offset from one."""
     return rms_scale(x, eps) * (1.0 + w)
 
 
@@ -60,7 +60,7 @@ def query_temperature(positions, coef, every):
 
 
 def softmax_attention(q, k, v, scale):
-    """One head over T tokens, causal: token i sees every j <= i. q, k [T, D]; v [T, V]."""
+    """One head over T tokens, causal: row i attends to rows 0 .. i. q, k [T, D]; v [T, V]."""
     T = q.shape[0]
     out = torch.zeros(T, v.shape[1], dtype=q.dtype)
     for i in range(T):
@@ -151,8 +151,8 @@ def glu_expert(h, gate, up, down):
 
 
 def choose_experts(scores, correction, top, groups, keep):
-    """For one token: the indices of the chosen experts, best first. Choice scores are the scores plus
-    the correction; a group of neighbours is worth the sum of its two largest choice scores (its only
+    """For one token: the indices of the chosen experts, best first. Selection values are the scores plus
+    the correction; a run of adjacent experts is worth the two highest of its selection values, added (its only
     one, if it has one expert); outside the `keep` best groups nothing can be chosen."""
     E = scores.shape[0]
     choice = scores + correction

@@ -291,7 +291,7 @@ def routed(logits, correction, E, top, groups, keep, width=None):
                                                        (40, 16, 16, 1, 1, -2.0), (70, 130, 7, 13, 4, -1.2), (1, 3, 3, 3, 3, 0.0),
                                                        (33, 9, 5, 3, 2, 0.7)])
 def test_choice_by_scores_within_groups(T, E, top, groups, keep, shift):
-    """Against the plain choice, token by token. With a correction around -1.5 every choice score is negative: an
+    """Against the plain choice, token by token. With a correction around -1.5 every selection value is negative: an
     expert outside the kept groups that counted as 0 instead of as minus infinity would then win."""
     logits, correction = rand(T, E, seed=E, scale=1.5), shift + 0.3 * rand(E, seed=top)
     routing = routed(logits, correction, E, top, groups, keep, width=E + 5)
@@ -323,7 +323,7 @@ def test_a_group_is_worth_its_two_best_and_the_correction_only_chooses():
     assert sorted(r.chosen.cpu().tolist()) == [0, 1]
     w = dict(zip(r.chosen.cpu().tolist(), r.weight.cpu()[0].tolist()))
     assert abs(w[0] - 0.9) < 1e-6 and abs(w[1] - 0.1) < 1e-6
-    # two groups kept of three, every choice score negative: the third group's experts are never taken
+    # two groups kept of three, every selection value negative: the third group's experts are never taken
     r = routed(logit([[0.3, 0.2, 0.6, 0.1, 0.5, 0.45]]), torch.full((6,), -2.0), 6, 4, 3, 2)
     assert sorted(r.chosen.cpu().tolist()) == [2, 3, 4, 5]
 

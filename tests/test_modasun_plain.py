@@ -105,7 +105,7 @@ def test_the_choice_of_experts():
     # two best, not all of a group and not the best alone
     assert sorted(plain.choose_experts(t(0.8, 0.1, 0.1, 0.5, 0.45, 0.4), torch.zeros(6, dtype=torch.float64), 2, 2, 1)) == [3, 4]
     assert sorted(plain.choose_experts(t(0.5, 0.45, 0.05, 0.4, 0.35, 0.34), torch.zeros(6, dtype=torch.float64), 2, 2, 1)) == [0, 1]
-    # the correction chooses; negative choice scores: the experts of other groups are out, not worth 0
+    # the correction chooses; negative selection values: the experts of other groups are out, not worth 0
     assert sorted(plain.choose_experts(t(0.9, 0.1, 0.6, 0.55), t(0.0, 0.5, 0.0, 0.0), 2, 2, 1)) == [0, 1]
     assert sorted(plain.choose_experts(t(0.3, 0.2, 0.6, 0.1, 0.5, 0.45), torch.full((6,), -2.0, dtype=torch.float64), 4, 3, 2)) == [2, 3, 4, 5]
     # groups of one expert are worth that expert
