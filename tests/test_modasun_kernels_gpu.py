@@ -186,7 +186,8 @@ def channel_delta_reference(proj, taps, z, a_log, dt_bias, kv_heads, heads, D, V
 
 
 @pytest.mark.parametrize("kv_heads,heads,D,V,K", [(1, 1, 8, 5, 1), (2, 6, 24, 70, 3), (3, 3, 48, 33, 4), (1, 2, 128, 64, 2),
-                                                  (2, 4, 32, 32, 3)])
+                                                  (2, 4, 32, 32, 3), (1, 2, 10, 12, 2), (2, 2, 34, 21, 3), (1, 3, 6, 7, 2),
+                                                  (1, 1, 160, 24, 2), (2, 2, 256, 16, 4)])
 def test_channel_decay_and_delta_rule_whole_in_portions_and_token_by_token(kv_heads, heads, D, V, K):
     C = 2 * kv_heads * D + heads * V
     ld = C + heads + 5
